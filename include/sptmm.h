@@ -1,0 +1,173 @@
+/*
+ * sptmm.h -- C ABI of the MI355X (gfx950) SpTMM engine.
+ *
+ * Multiplication-free ternary-weight sparse matrix multiply
+ *     C[m][n] = sum_{k in pos(n)} X[m][k] - sum_{k in neg(n)} X[m][k]
+ * with three encodings of the same ternary K x N matrix W:
+ *   u16    row-index lists per column (reference "SpTMM",       -row_split3_small)
+ *   delta  8/16-bit gaps of the sorted lists (reference "SpTMM-delta", -row_split_delta2)
+ *   i2s    2-bit packed dense ternary, 16 weights per 32-bit word (reference -i2s)
+ *
+ * Plain pointers and sizes only; no HIP or torch types.  `stream` arguments are
+ * a hipStream_t passed as void* (NULL = the default stream).  Every function
+ * returns SPTMM_OK (0) or a negative sptmm_status; sptmm_last_error() gives the
+ * text of the last failure on the calling thread.  The library never exits or
+ * aborts.  Calls on one sptmm_weights object from several threads are safe as
+ * long as each uses its own X/C buffers (the object is immutable after upload).
+ *
+ * The reference has no library boundary of its own: its only interface is the
+ * `rcr` command line plus the kernels' argument lists.  Each entry point below
+ * names the reference code (file:line under the reference checkout) it stands
+ * in for.
+ */
+#ifndef SPTMM_H
+#define SPTMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum sptmm_status {
+    SPTMM_OK = 0,
+    SPTMM_ERR_INVALID = -1,     /* argument or shape violates a documented rule   */
+    SPTMM_ERR_UNSUPPORTED = -2, /* valid request this build cannot serve          */
+    SPTMM_ERR_HIP = -3,         /* a HIP runtime call failed (see last_error)     */
+    SPTMM_ERR_NOMEM = -4
+} sptmm_status;
+
+typedef enum sptmm_kind { SPTMM_KIND_U16 = 1, SPTMM_KIND_DELTA = 2, SPTMM_KIND_I2S = 3 } sptmm_kind;
+
+typedef struct sptmm_devinfo {
+    char name[128];
+    char arch[64];
+    int compute_units;
+    int wave_size;
+    int lds_bytes_per_workgroup; /* largest LDS allocation one workgroup may make */
+    int l2_bytes;
+    uint64_t hbm_bytes;
+    double peak_hbm_gbps;        /* published peak used for roofline lines (8000 on MI355X) */
+} sptmm_devinfo;
+
+typedef struct sptmm_winfo {
+    int kind;        /* sptmm_kind */
+    int K, N, S;     /* S = nonzeros per column (0 for i2s) */
+    int split_k;     /* lanes cooperating on one column (0 for i2s) */
+    int delta_bits;  /* 8 or 16 for SPTMM_KIND_DELTA, else 0 */
+    uint64_t stream_bytes; /* bytes of the weight stream one GEMV reads */
+} sptmm_winfo;
+
+typedef struct sptmm_weights sptmm_weights; /* opaque; owns its device buffer */
+
+const char *sptmm_last_error(void);
+const char *sptmm_version(void);
+
+/* ------------------------------------------------------------------ host side
+ * Weight generator and format builders.  Pure host code (no GPU needed). */
+
+/* Seeded ternary matrix of the benchmark: main.cu:246-276 (generator + sorted
+ * +1/-1 row lists) with the RNG of macro.cuh:69-76.  pos/neg are [N][S/2];
+ * W_colmajor (K*N bytes, column n at W + n*K) may be NULL.
+ * Rules of main.cu:85-91: K,N multiples of 16, K < 65536, S even, K > S. */
+int sptmm_generate_ternary(int K, int N, int S, int8_t *W_colmajor, uint16_t *pos, uint16_t *neg);
+
+/* Row lists of an arbitrary balanced ternary matrix (exactly S/2 of each sign
+ * per column, as main.cu:276 asserts). */
+int sptmm_lists_from_dense(const int8_t *W_colmajor, int K, int N, int S, uint16_t *pos, uint16_t *neg);
+
+/* Seeded int8 activations, uniform on [-127,127] (stands in for make_X,
+ * main.cu:784-797, which is unseeded): xorshift32 stream, r % 255 - 127. */
+int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X);
+
+/* Wave64 stream of the u16 lists; replaces the W_map_{8,16,32}_div layouts of
+ * main.cu:343-374.  split_k in {8,16,32,64,128,256}; (S/2) % split_k == 0
+ * (main.cu:564). */
+size_t sptmm_pack_u16_bytes(int N, int S, int split_k);
+int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out);
+int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg);
+
+/* Gap streams; replaces W_map_delta2_d / W_map_delta2_div256 of main.cu:376-413.
+ * Each lane owns a contiguous run of the sorted list: a 16-bit restart index
+ * followed by its gaps.  sptmm_delta_bits() returns 8 when every in-run gap
+ * fits a byte, else 16 (the reference narrows silently, main.cu:380-383).
+ * split_k in {8,16,32,64}. */
+int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int split_k);
+size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits);
+int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out);
+int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg);
+
+/* i2s: 16 weights per word, code = w + 2, element e at bit 8*(e%4) + 2*(e/4)
+ * (main.cu:176-192, decode bitnet_kernels.cuh:52-72).  Word order is this
+ * library's own wave64 tiling, not the reference's (whose prepared matrix,
+ * main.cu:194-196, does not match its kernel's addressing anyway). */
+uint32_t sptmm_i2s_pack_word(const int8_t w16[16]);
+void sptmm_i2s_decode_word(uint32_t word, int8_t w16[16]);
+size_t sptmm_pack_i2s_bytes(int K, int N);
+int sptmm_pack_i2s(const int8_t *W_colmajor, int K, int N, void *out);
+int sptmm_unpack_i2s(const void *packed, int K, int N, int8_t *W_colmajor);
+
+/* ---------------------------------------------------------------- device side */
+
+/* Selects the device and reports what the roofline lines need. */
+int sptmm_device_init(int device, sptmm_devinfo *out);
+
+/* Host lists / dense matrix -> device stream.  Stand in for the cudaMalloc +
+ * prepareW_map / prepareW_i2s sequence of main.cu:914-989 and 1851-1859. */
+int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
+int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
+int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weights **out);
+/* Second device copy of the same stream (used to rotate over more bytes than
+ * the last-level cache holds when timing cold reads). */
+int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out);
+void sptmm_weights_free(sptmm_weights *w);
+int sptmm_weights_info(const sptmm_weights *w, sptmm_winfo *out);
+size_t sptmm_weights_bytes(const sptmm_weights *w);
+
+/* C[M][N] = X[M][K] . W, X and C row-major device pointers (main.cu:575,592).
+ * Asynchronous on `stream`.
+ *   sptmm_gemv_i8  int8 activations, exact int32 sums: rowWiseSplit3Small4
+ *                  (main.cu:556-594), rowWiseSplit2DeltaSmallAsync2/3
+ *                  (main.cu:599-764) or ladder_int8xint2_kernel
+ *                  (bitnet_kernels.cuh:75-111), by the kind of `w`.
+ *   sptmm_gemv_f16 fp16 activations (raw bits), fp32 sums; u16 and delta kinds.
+ *   sptmm_gemv_f32 fp32 activations, fp32 sums; u16 and delta kinds. */
+int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X_dev, int M, int32_t *C_dev, void *stream);
+int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X_dev, int M, float *C_dev, void *stream);
+int sptmm_gemv_f32(const sptmm_weights *w, const float *X_dev, int M, float *C_dev, void *stream);
+
+/* Thin device-memory / stream / event helpers so callers need no HIP headers
+ * (the cudaMalloc/cudaMemcpy/cudaEvent* calls of main.cu:767-782, 804-815). */
+int sptmm_malloc(void **dev_ptr, size_t bytes);
+int sptmm_free(void *dev_ptr);
+int sptmm_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
+int sptmm_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
+int sptmm_memset(void *dst_dev, int value, size_t bytes);
+int sptmm_stream_create(void **stream);
+int sptmm_stream_destroy(void *stream);
+int sptmm_stream_sync(void *stream);
+int sptmm_device_sync(void);
+int sptmm_event_create(void **event);
+int sptmm_event_destroy(void *event);
+int sptmm_event_record(void *event, void *stream);
+int sptmm_event_sync(void *event);
+int sptmm_event_elapsed_us(void *start, void *stop, double *us);
+/* The timing loop of measureKernel (main.cu:767-782) around `iters` GEMV
+ * launches, kept native so that no interpreter sits between launches.  Launch i
+ * uses ws[i % n_ws] (several device copies of one matrix defeat the last-level
+ * cache).  act: 0 int8, 1 fp16, 2 fp32.  mode: 0 = back-to-back launches on one
+ * stream between two events; 1 = stream synchronize after every launch, as the
+ * reference does (main.cu:1456); 2 = one rotation captured into a HIP graph and
+ * replayed.  Reports mean microseconds per launch. */
+int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X_dev, int M, void *C_dev,
+                       int iters, int mode, double *us_per_call);
+/* Reads `bytes` of a scratch buffer and writes them back (a plain copy kernel):
+ * evicts cached weight streams between cold-read timings and calibrates the
+ * traffic counters. */
+int sptmm_copy_kernel(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPTMM_H */

@@ -1,0 +1,383 @@
+"""ctypes binding of include/sptmm.h (libsptmm.so, built in-tree by sptmm_amd.build)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+__all__ = [
+    "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
+    "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s",
+    "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel",
+    "device_sync", "measure_gemv", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
+]
+
+KIND_U16, KIND_DELTA, KIND_I2S = 1, 2, 3
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+# every symbol include/sptmm.h declares
+EXPORTS = [
+    "sptmm_last_error", "sptmm_version", "sptmm_generate_ternary", "sptmm_lists_from_dense", "sptmm_make_x_i8",
+    "sptmm_pack_u16_bytes", "sptmm_pack_u16", "sptmm_unpack_u16", "sptmm_delta_bits", "sptmm_pack_delta_bytes",
+    "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
+    "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_device_init",
+    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_i2s", "sptmm_weights_clone",
+    "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
+    "sptmm_gemv_f32", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
+    "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
+    "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
+    "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel",
+]
+
+
+class SptmmError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("sptmm error %d: %s" % (code, msg))
+        self.code = code
+
+
+class DevInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int),
+                ("wave_size", C.c_int), ("lds_bytes_per_workgroup", C.c_int), ("l2_bytes", C.c_int),
+                ("hbm_bytes", C.c_uint64), ("peak_hbm_gbps", C.c_double)]
+
+
+class WInfo(C.Structure):
+    _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
+                ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64)]
+
+
+def lib_path() -> str:
+    return os.path.join(_PKG, "libsptmm.so")
+
+
+def lib() -> C.CDLL:
+    """The HIP library.  Raises if it has not been built: there is no fallback path."""
+    global _LIB
+    if _LIB is None:
+        p = lib_path()
+        if not os.path.exists(p):
+            raise RuntimeError("%s is missing: build it with `python -m sptmm_amd.build` "
+                               "(hipcc --offload-arch=gfx950); there is no CPU fallback" % p)
+        L = C.CDLL(p)
+        L.sptmm_last_error.restype = C.c_char_p
+        L.sptmm_version.restype = C.c_char_p
+        for n in ("sptmm_pack_u16_bytes", "sptmm_pack_delta_bytes", "sptmm_pack_i2s_bytes", "sptmm_weights_bytes"):
+            getattr(L, n).restype = C.c_size_t
+        L.sptmm_i2s_pack_word.restype = C.c_uint32
+        L.sptmm_i2s_decode_word.restype = None
+        L.sptmm_weights_free.restype = None
+        L.sptmm_weights_free.argtypes = [C.c_void_p]
+        L.sptmm_weights_bytes.argtypes = [C.c_void_p]
+        L.sptmm_weights_info.argtypes = [C.c_void_p, C.POINTER(WInfo)]
+        L.sptmm_weights_clone.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        for n in ("sptmm_gemv_i8", "sptmm_gemv_f16", "sptmm_gemv_f32"):
+            getattr(L, n).argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.sptmm_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        L.sptmm_free.argtypes = [C.c_void_p]
+        L.sptmm_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.sptmm_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.sptmm_memset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+        L.sptmm_measure_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                         C.c_int, C.POINTER(C.c_double)]
+        L.sptmm_copy_kernel.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.sptmm_make_x_i8.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p]
+        for n in ("sptmm_stream_create", "sptmm_event_create"):
+            getattr(L, n).argtypes = [C.POINTER(C.c_void_p)]
+        for n in ("sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_event_destroy", "sptmm_event_sync"):
+            getattr(L, n).argtypes = [C.c_void_p]
+        L.sptmm_event_record.argtypes = [C.c_void_p, C.c_void_p]
+        L.sptmm_event_elapsed_us.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]
+        _LIB = L
+    return _LIB
+
+
+def _ck(rc: int) -> int:
+    if rc < 0:
+        raise SptmmError(rc, lib().sptmm_last_error().decode())
+    return rc
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert isinstance(a, np.ndarray) and a.flags["C_CONTIGUOUS"], "need a C-contiguous numpy array"
+    return a.ctypes.data_as(C.c_void_p)
+
+
+# ------------------------------------------------------------------ host side
+def device_init(device: int = 0) -> dict:
+    info = DevInfo()
+    _ck(lib().sptmm_device_init(device, C.byref(info)))
+    return {f: (getattr(info, f).decode() if isinstance(getattr(info, f), bytes) else getattr(info, f))
+            for f, _ in DevInfo._fields_}
+
+
+def generate_ternary(K: int, N: int, S: int, dense: bool = False):
+    """-> (W [N][K] int8 = column-major K x N, or None; pos [N][S/2] u16; neg [N][S/2] u16)."""
+    half = max(S // 2, 0)
+    W = np.empty((N, K), np.int8) if dense and K > 0 and N > 0 else None
+    pos = np.empty((max(N, 0), half), np.uint16)
+    neg = np.empty((max(N, 0), half), np.uint16)
+    _ck(lib().sptmm_generate_ternary(K, N, S, _p(W), _p(pos), _p(neg)))
+    return W, pos, neg
+
+
+def lists_from_dense(W: np.ndarray, S: int):
+    N, K = W.shape
+    pos = np.empty((N, S // 2), np.uint16)
+    neg = np.empty((N, S // 2), np.uint16)
+    _ck(lib().sptmm_lists_from_dense(_p(W), K, N, S, _p(pos), _p(neg)))
+    return pos, neg
+
+
+def make_x_i8(seed: int, M: int, K: int) -> np.ndarray:
+    X = np.empty((M, K), np.int8)
+    _ck(lib().sptmm_make_x_i8(seed, M * K, _p(X)))
+    return X
+
+
+def pack_u16(pos, neg, K, split_k) -> np.ndarray:
+    N, half = pos.shape
+    n = lib().sptmm_pack_u16_bytes(N, 2 * half, split_k)
+    out = np.zeros(max(n, 1), np.uint8)
+    _ck(lib().sptmm_pack_u16(_p(pos), _p(neg), K, N, 2 * half, split_k, _p(out)))
+    return out[:n]
+
+
+def unpack_u16(packed, K, N, S, split_k):
+    pos = np.empty((N, S // 2), np.uint16)
+    neg = np.empty((N, S // 2), np.uint16)
+    _ck(lib().sptmm_unpack_u16(_p(packed), K, N, S, split_k, _p(pos), _p(neg)))
+    return pos, neg
+
+
+def delta_bits(pos, neg, split_k) -> int:
+    N, half = pos.shape
+    return _ck(lib().sptmm_delta_bits(_p(pos), _p(neg), N, 2 * half, split_k))
+
+
+def pack_delta(pos, neg, K, split_k, bits=None) -> tuple[np.ndarray, int]:
+    N, half = pos.shape
+    if bits is None:
+        bits = delta_bits(pos, neg, split_k)
+    n = lib().sptmm_pack_delta_bytes(N, 2 * half, split_k, bits)
+    out = np.zeros(max(n, 1), np.uint8)
+    _ck(lib().sptmm_pack_delta(_p(pos), _p(neg), K, N, 2 * half, split_k, bits, _p(out)))
+    return out[:n], bits
+
+
+def unpack_delta(packed, K, N, S, split_k, bits):
+    pos = np.empty((N, S // 2), np.uint16)
+    neg = np.empty((N, S // 2), np.uint16)
+    _ck(lib().sptmm_unpack_delta(_p(packed), K, N, S, split_k, bits, _p(pos), _p(neg)))
+    return pos, neg
+
+
+def i2s_pack_word(w16) -> int:
+    a = np.ascontiguousarray(w16, np.int8)
+    assert a.size == 16
+    return int(lib().sptmm_i2s_pack_word(_p(a)))
+
+
+def i2s_decode_word(word: int) -> np.ndarray:
+    out = np.empty(16, np.int8)
+    lib().sptmm_i2s_decode_word(C.c_uint32(word), _p(out))
+    return out
+
+
+def pack_i2s(W: np.ndarray) -> np.ndarray:
+    N, K = W.shape
+    n = lib().sptmm_pack_i2s_bytes(K, N)
+    out = np.zeros(max(n, 1), np.uint8)
+    _ck(lib().sptmm_pack_i2s(_p(W), K, N, _p(out)))
+    return out[:n]
+
+
+def unpack_i2s(packed, K, N) -> np.ndarray:
+    W = np.empty((N, K), np.int8)
+    _ck(lib().sptmm_unpack_i2s(_p(packed), K, N, _p(W)))
+    return W
+
+
+# ---------------------------------------------------------------- device side
+class DeviceBuffer:
+    """A device allocation owned through the C ABI."""
+
+    def __init__(self, nbytes: int):
+        self.ptr = C.c_void_p()
+        self.nbytes = int(nbytes)
+        _ck(lib().sptmm_malloc(C.byref(self.ptr), self.nbytes))
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        if a.nbytes:
+            _ck(lib().sptmm_memcpy_h2d(b.ptr, _p(a), a.nbytes))
+        return b
+
+    def to_numpy(self, dtype, shape) -> np.ndarray:
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        if out.nbytes:
+            _ck(lib().sptmm_memcpy_d2h(_p(out), self.ptr, out.nbytes))
+        return out
+
+    def fill(self, byte: int = 0):
+        _ck(lib().sptmm_memset(self.ptr, byte, self.nbytes))
+
+    def free(self):
+        if self.ptr:
+            lib().sptmm_free(self.ptr)
+            self.ptr = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Stream:
+    def __init__(self):
+        self.handle = C.c_void_p()
+        _ck(lib().sptmm_stream_create(C.byref(self.handle)))
+
+    def sync(self):
+        _ck(lib().sptmm_stream_sync(self.handle))
+
+    def destroy(self):
+        if self.handle:
+            lib().sptmm_stream_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+
+class Event:
+    def __init__(self):
+        self.handle = C.c_void_p()
+        _ck(lib().sptmm_event_create(C.byref(self.handle)))
+
+    def record(self, stream: Stream | None = None):
+        _ck(lib().sptmm_event_record(self.handle, stream.handle if stream else None))
+
+    def sync(self):
+        _ck(lib().sptmm_event_sync(self.handle))
+
+    def elapsed_us(self, later: "Event") -> float:
+        us = C.c_double()
+        _ck(lib().sptmm_event_elapsed_us(self.handle, later.handle, C.byref(us)))
+        return us.value
+
+    def destroy(self):
+        if self.handle:
+            lib().sptmm_event_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+
+def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuffer", iters: int, mode: int = 0) -> float:
+    """Mean microseconds per launch over `iters` launches rotating over `weights` (see sptmm_measure_gemv)."""
+    arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
+    us = C.c_double()
+    _ck(lib().sptmm_measure_gemv(arr, len(weights), act, X.ptr, M, Cout.ptr, iters, mode, C.byref(us)))
+    return us.value
+
+
+def device_sync():
+    _ck(lib().sptmm_device_sync())
+
+
+def copy_kernel(dst: DeviceBuffer, src: DeviceBuffer, nbytes: int, stream: Stream | None = None):
+    _ck(lib().sptmm_copy_kernel(dst.ptr, src.ptr, nbytes, stream.handle if stream else None))
+
+
+class Weights:
+    """One ternary K x N matrix resident on the device in one of the three encodings."""
+
+    def __init__(self, handle):
+        self.handle = handle
+
+    @classmethod
+    def upload_u16(cls, pos, neg, K, split_k) -> "Weights":
+        N, half = pos.shape
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_upload_u16(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def upload_delta(cls, pos, neg, K, split_k) -> "Weights":
+        N, half = pos.shape
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_upload_delta(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def upload_i2s(cls, W: np.ndarray) -> "Weights":
+        N, K = W.shape
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_upload_i2s(_p(W), K, N, C.byref(h)))
+        return cls(h)
+
+    def clone(self) -> "Weights":
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_clone(self.handle, C.byref(h)))
+        return Weights(h)
+
+    @property
+    def info(self) -> dict:
+        wi = WInfo()
+        _ck(lib().sptmm_weights_info(self.handle, C.byref(wi)))
+        return {f: getattr(wi, f) for f, _ in WInfo._fields_}
+
+    @property
+    def nbytes(self) -> int:
+        return int(lib().sptmm_weights_bytes(self.handle))
+
+    # raw launches on device buffers (asynchronous on `stream`)
+    def gemv_i8(self, X: DeviceBuffer, M: int, Cout: DeviceBuffer, stream: Stream | None = None):
+        _ck(lib().sptmm_gemv_i8(self.handle, X.ptr, M, Cout.ptr, stream.handle if stream else None))
+
+    def gemv_f16(self, X: DeviceBuffer, M: int, Cout: DeviceBuffer, stream: Stream | None = None):
+        _ck(lib().sptmm_gemv_f16(self.handle, X.ptr, M, Cout.ptr, stream.handle if stream else None))
+
+    def gemv_f32(self, X: DeviceBuffer, M: int, Cout: DeviceBuffer, stream: Stream | None = None):
+        _ck(lib().sptmm_gemv_f32(self.handle, X.ptr, M, Cout.ptr, stream.handle if stream else None))
+
+    def matmul(self, X: np.ndarray) -> np.ndarray:
+        """Host convenience: upload X [M][K], run on the device, download C [M][N]."""
+        i = self.info
+        M, K = X.shape
+        assert K == i["K"]
+        xb = DeviceBuffer.from_numpy(X)
+        cb = DeviceBuffer(4 * M * i["N"])
+        cb.fill(0xFF)
+        try:
+            if X.dtype == np.int8:
+                self.gemv_i8(xb, M, cb)
+                out = np.int32
+            elif X.dtype == np.float16:
+                self.gemv_f16(xb, M, cb)
+                out = np.float32
+            elif X.dtype == np.float32:
+                self.gemv_f32(xb, M, cb)
+                out = np.float32
+            else:
+                raise TypeError("activations must be int8, float16 or float32")
+            device_sync()
+            return cb.to_numpy(out, (M, i["N"]))
+        finally:
+            xb.free()
+            cb.free()
+
+    def free(self):
+        if self.handle:
+            lib().sptmm_weights_free(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass

@@ -1,0 +1,386 @@
+// Host side of the SpTMM engine: seeded weight generator and the builders of
+// the three device streams.  Pure C++ (no GPU), so it is unit-testable on any
+// machine.  The streams are laid out for 64-lane wavefronts: every per-lane
+// load of a wavefront touches one contiguous, naturally aligned block.
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+#include "internal.hpp"
+
+namespace sptmm {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_shape(int K, int N, int S)
+{
+    // main.cu:85-91
+    if (K <= 0 || N <= 0 || S <= 0) return fail(SPTMM_ERR_INVALID, "K, N and S must be positive");
+    if (K % 16) return fail(SPTMM_ERR_INVALID, "K mod 16 should be 0");
+    if (N % 16) return fail(SPTMM_ERR_INVALID, "N mod 16 should be 0");
+    if (K >= 65536) return fail(SPTMM_ERR_INVALID, "K should fit an unsigned 16-bit row index");
+    if (S % 2) return fail(SPTMM_ERR_INVALID, "S mod 2 must be 0 so that the +1 and -1 lists have the same size");
+    if (K <= S) return fail(SPTMM_ERR_INVALID, "K should be bigger than S");
+    return SPTMM_OK;
+}
+
+int make_geometry(int N, int S, int split_k, int max_split, Geometry *g)
+{
+    bool ok = false;
+    for (int s = 8; s <= max_split; s *= 2) ok |= (s == split_k);
+    if (!ok) return fail(SPTMM_ERR_INVALID, "Wrong split size");
+    int half = S / 2;
+    if (half % split_k) return fail(SPTMM_ERR_INVALID, "Wrong SPLIT Size: (S/2) %% split_k != 0");
+    g->N = N;
+    g->half = half;
+    g->split_k = split_k;
+    g->L = std::min(split_k, 64);
+    g->G = 64 / g->L;
+    g->W = std::max(1, split_k / 64);
+    g->n_lane = half / split_k;
+    if (N % g->G) return fail(SPTMM_ERR_INVALID, "N must be a multiple of %d for split_k=%d", g->G, split_k);
+    g->tasks = N / g->G * g->W;
+    return SPTMM_OK;
+}
+
+size_t slot_offset(int n_lane, int esz, int sign, int lane, int j)
+{
+    const int e16 = 16 / esz;
+    const int full = n_lane / e16;
+    if (j < full * e16) return (size_t)(j / e16) * 2048 + (size_t)sign * 1024 + (size_t)lane * 16 + (size_t)(j % e16) * esz;
+    size_t base = (size_t)full * 2048;
+    int rem = n_lane - full * e16, first = full * e16;
+    for (int w = 8; w >= esz; w /= 2) {
+        int cnt = w / esz;
+        if (rem & cnt) {
+            if (j < first + cnt) return base + (size_t)sign * 64 * w + (size_t)lane * w + (size_t)(j - first) * esz;
+            first += cnt;
+            base += (size_t)128 * w;
+        }
+    }
+    return (size_t)-1;  // unreachable for j < n_lane
+}
+
+// Which (task, lane, slot) holds entry i of column c.  u16 lists interleave a
+// column over its split_k lanes (entry i -> lane i % split_k, the assignment of
+// main.cu:343-374); gap streams give each lane a contiguous run.
+struct Place {
+    int task, lane, slot;
+};
+static inline Place place(const Geometry &g, int c, int i, bool contiguous)
+{
+    int v = contiguous ? i / g.n_lane : i % g.split_k;  // virtual lane 0..split_k-1
+    int slot = contiguous ? i % g.n_lane : i / g.split_k;
+    Place p;
+    if (g.W > 1) {
+        p.task = c * g.W + v / 64;
+        p.lane = v % 64;
+    } else {
+        p.task = c / g.G;
+        p.lane = (c % g.G) * g.L + v;
+    }
+    p.slot = slot;
+    return p;
+}
+
+template <class F>
+static void parallel_columns(int N, F f)
+{
+    unsigned hw = std::thread::hardware_concurrency();
+    int nt = (int)std::min<unsigned>(hw ? hw : 1, 16);
+    if (N < 64) nt = 1;
+    std::vector<std::thread> th;
+    for (int t = 0; t < nt; ++t)
+        th.emplace_back([=] {
+            int c0 = (int)((long)N * t / nt), c1 = (int)((long)N * (t + 1) / nt);
+            for (int c = c0; c < c1; ++c) f(c);
+        });
+    for (auto &t : th) t.join();
+}
+
+static inline uint32_t xorshift32(uint32_t &s)
+{
+    s ^= s << 13;
+    s ^= s >> 17;
+    s ^= s << 5;
+    return s;
+}
+
+}  // namespace sptmm
+
+using namespace sptmm;
+
+extern "C" {
+
+const char *sptmm_last_error(void) { return g_err; }
+const char *sptmm_version(void) { return "sptmm-mi355x 0.1 (gfx950)"; }
+
+int sptmm_lists_from_dense(const int8_t *W, int K, int N, int S, uint16_t *pos, uint16_t *neg)
+{
+    if (int rc = check_shape(K, N, S)) return rc;
+    if (!W || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const int half = S / 2;
+    std::vector<int> bad(N, 0);
+    parallel_columns(N, [&](int c) {
+        const int8_t *w = W + (size_t)c * K;
+        int np = 0, nn = 0;
+        for (int r = 0; r < K; ++r) {
+            if (w[r] == 1) {
+                if (np < half) pos[(size_t)c * half + np] = (uint16_t)r;
+                ++np;
+            } else if (w[r] == -1) {
+                if (nn < half) neg[(size_t)c * half + nn] = (uint16_t)r;
+                ++nn;
+            } else if (w[r] != 0) {
+                bad[c] = 1;
+            }
+        }
+        if (np != half || nn != half) bad[c] = 1;
+    });
+    for (int c = 0; c < N; ++c)
+        if (bad[c]) return fail(SPTMM_ERR_INVALID, "W matrix corrupt: column %d is not ternary with S/2 entries per sign", c);
+    return SPTMM_OK;
+}
+
+int sptmm_generate_ternary(int K, int N, int S, int8_t *W, uint16_t *pos, uint16_t *neg)
+{
+    if (int rc = check_shape(K, N, S)) return rc;
+    if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const int half = S / 2;
+    parallel_columns(N, [&](int c) {
+        std::vector<int8_t> local;
+        int8_t *w;
+        if (W) {
+            w = W + (size_t)c * K;
+        } else {
+            local.resize(K);
+            w = local.data();
+        }
+        std::fill(w, w + half, (int8_t)-1);
+        std::fill(w + half, w + S, (int8_t)1);
+        std::fill(w + S, w + K, (int8_t)0);
+        uint32_t st = 0xCAFEBABEu ^ (uint32_t)c;
+        for (uint32_t i = (uint32_t)K - 1; i > 0; --i) std::swap(w[i], w[xorshift32(st) % (i + 1)]);
+        uint16_t *p = pos + (size_t)c * half, *q = neg + (size_t)c * half;
+        for (int r = 0; r < K; ++r) {
+            if (w[r] > 0) *p++ = (uint16_t)r;
+            if (w[r] < 0) *q++ = (uint16_t)r;
+        }
+    });
+    return SPTMM_OK;
+}
+
+int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X)
+{
+    if (!X) return fail(SPTMM_ERR_INVALID, "null pointer");
+    uint32_t st = seed ? seed : 1u;
+    for (size_t i = 0; i < count; ++i) X[i] = (int8_t)((int)(xorshift32(st) % 255u) - 127);
+    return SPTMM_OK;
+}
+
+// ------------------------------------------------------------------ u16 stream
+size_t sptmm_pack_u16_bytes(int N, int S, int split_k)
+{
+    Geometry g;
+    if (make_geometry(N, S, split_k, 256, &g)) return 0;
+    return (size_t)g.tasks * 256 * g.n_lane;
+}
+
+static int u16_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int K, int N, int S, int split_k)
+{
+    if (int rc = check_shape(K, N, S)) return rc;
+    Geometry g;
+    if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
+    if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const size_t task_bytes = (size_t)256 * g.n_lane;
+    uint8_t *base = (uint8_t *)packed;
+    parallel_columns(N, [&](int c) {
+        for (int sign = 0; sign < 2; ++sign) {
+            uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
+            for (int i = 0; i < g.half; ++i) {
+                Place p = place(g, c, i, false);
+                uint16_t *cell = (uint16_t *)(base + p.task * task_bytes + slot_offset(g.n_lane, 2, sign, p.lane, p.slot));
+                if (pack)
+                    *cell = lst[i];
+                else
+                    lst[i] = *cell;
+            }
+        }
+    });
+    return SPTMM_OK;
+}
+
+int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out)
+{
+    if (pos && neg)
+        for (size_t i = 0, n = (size_t)N * (S / 2); i < n; ++i)
+            if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
+    return u16_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k);
+}
+
+int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg)
+{
+    return u16_walk(false, (void *)packed, pos, neg, K, N, S, split_k);
+}
+
+// ---------------------------------------------------------------- gap streams
+// Task layout: 256-byte header of restart indices, u16 [sign][lane], then the
+// gap rounds.  The first gap of every run is stored as 0 (the restart index is
+// the run's first row), so a lane's walk is "idx = restart; idx += gap; gather".
+int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int split_k)
+{
+    Geometry g;
+    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
+    if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    for (int sign = 0; sign < 2; ++sign) {
+        const uint16_t *l = sign ? neg : pos;
+        for (int c = 0; c < N; ++c)
+            for (int i = 1; i < g.half; ++i) {
+                if (i % g.n_lane == 0) continue;  // run start: absolute
+                size_t o = (size_t)c * g.half + i;
+                if (l[o] <= l[o - 1]) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending");
+                if (l[o] - l[o - 1] > 255) return 16;
+            }
+    }
+    return 8;
+}
+
+size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits)
+{
+    Geometry g;
+    if (make_geometry(N, S, split_k, 64, &g)) return 0;
+    if (bits != 8 && bits != 16) return 0;
+    return (size_t)g.tasks * (256 + (size_t)64 * 2 * g.n_lane * (bits / 8));
+}
+
+static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int K, int N, int S, int split_k, int bits)
+{
+    if (int rc = check_shape(K, N, S)) return rc;
+    Geometry g;
+    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
+    if (bits != 8 && bits != 16) return fail(SPTMM_ERR_INVALID, "delta bits must be 8 or 16");
+    if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const int esz = bits / 8;
+    const size_t task_bytes = 256 + (size_t)128 * g.n_lane * esz;
+    uint8_t *base = (uint8_t *)packed;
+    std::vector<int> bad(N, 0);
+    parallel_columns(N, [&](int c) {
+        for (int sign = 0; sign < 2; ++sign) {
+            uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
+            unsigned run = 0;
+            for (int i = 0; i < g.half; ++i) {
+                Place p = place(g, c, i, true);
+                uint8_t *task = base + p.task * task_bytes;
+                uint16_t *restart = (uint16_t *)(task + sign * 128 + p.lane * 2);
+                uint8_t *cell = task + 256 + slot_offset(g.n_lane, esz, sign, p.lane, p.slot);
+                if (pack) {
+                    unsigned gap = 0;
+                    if (p.slot == 0) {
+                        *restart = lst[i];
+                    } else {
+                        gap = (unsigned)lst[i] - lst[i - 1];
+                        if (lst[i] <= lst[i - 1] || gap >= (1u << bits)) bad[c] = 1;
+                    }
+                    if (esz == 1)
+                        *cell = (uint8_t)gap;
+                    else
+                        *(uint16_t *)cell = (uint16_t)gap;
+                } else {
+                    unsigned gap = esz == 1 ? *cell : *(uint16_t *)cell;
+                    run = p.slot == 0 ? *restart + gap : run + gap;
+                    lst[i] = (uint16_t)run;
+                }
+            }
+        }
+    });
+    for (int c = 0; c < N; ++c)
+        if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d: list not ascending or gap does not fit %d bits", c, bits);
+    return SPTMM_OK;
+}
+
+int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out)
+{
+    if (pos && neg)
+        for (size_t i = 0, n = (size_t)N * (S / 2); i < n; ++i)
+            if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
+    return delta_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k, bits);
+}
+
+int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg)
+{
+    return delta_walk(false, (void *)packed, pos, neg, K, N, S, split_k, bits);
+}
+
+// ------------------------------------------------------------------------ i2s
+uint32_t sptmm_i2s_pack_word(const int8_t w16[16])
+{
+    uint32_t word = 0;
+    for (int e = 0; e < 16; ++e) word |= ((uint32_t)(w16[e] + 2) & 3u) << (8 * (e & 3) + 2 * (e >> 2));
+    return word;
+}
+
+void sptmm_i2s_decode_word(uint32_t word, int8_t w16[16])
+{
+    for (int e = 0; e < 16; ++e) w16[e] = (int8_t)((int)((word >> (8 * (e & 3) + 2 * (e >> 2))) & 3u) - 2);
+}
+
+size_t sptmm_pack_i2s_bytes(int K, int N)
+{
+    if (K <= 0 || N <= 0 || K % 16 || N % 16) return 0;
+    return (size_t)N * i2s_padded_k(K) / 4;
+}
+
+// Word index of rows [16*g16, 16*g16+16) of column c: tiles of 16 columns x 256
+// rows (1 KiB); inside a tile lane = (c%16)*4 + quarter, 4 words per lane.
+static inline size_t i2s_word_index(int Kp, int c, int g16)
+{
+    int rounds = Kp / 256, r = g16 / 16, q = (g16 % 16) / 4, j = g16 % 4;
+    return ((size_t)(c / 16) * rounds + r) * 256 + (size_t)((c % 16) * 4 + q) * 4 + j;
+}
+
+int sptmm_pack_i2s(const int8_t *W, int K, int N, void *out)
+{
+    if (K <= 0 || N <= 0 || K % 16 || N % 16) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
+    if (!W || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const int Kp = i2s_padded_k(K);
+    uint32_t *o = (uint32_t *)out;
+    std::vector<int> bad(N, 0);
+    parallel_columns(N, [&](int c) {
+        for (int g16 = 0; g16 < Kp / 16; ++g16) {
+            int8_t w16[16] = {0};
+            if (g16 * 16 < K) {
+                memcpy(w16, W + (size_t)c * K + 16 * g16, 16);
+                for (int e = 0; e < 16; ++e)
+                    if (w16[e] < -1 || w16[e] > 1) bad[c] = 1;
+            }
+            o[i2s_word_index(Kp, c, g16)] = sptmm_i2s_pack_word(w16);
+        }
+    });
+    for (int c = 0; c < N; ++c)
+        if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d holds a weight outside {-1,0,1}", c);
+    return SPTMM_OK;
+}
+
+int sptmm_unpack_i2s(const void *packed, int K, int N, int8_t *W)
+{
+    if (K <= 0 || N <= 0 || K % 16 || N % 16) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
+    if (!W || !packed) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const int Kp = i2s_padded_k(K);
+    const uint32_t *p = (const uint32_t *)packed;
+    for (int c = 0; c < N; ++c)
+        for (int g16 = 0; g16 < K / 16; ++g16) sptmm_i2s_decode_word(p[i2s_word_index(Kp, c, g16)], W + (size_t)c * K + 16 * g16);
+    return SPTMM_OK;
+}
+
+}  // extern "C"

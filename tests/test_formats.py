@@ -1,0 +1,161 @@
+"""Host logic of the library (generator, stream builders) -- no GPU needed.
+
+The library's own generator is compared with the oracle's restatement of
+main.cu:246-276; the three device streams are checked as bijections of the row
+lists / dense matrix, against closed-form offset formulas, and through
+pack -> unpack round trips.
+"""
+import numpy as np
+import pytest
+
+import oracle
+import sptmm_amd as sp
+
+SHAPES = [(64, 16, 32), (512, 32, 256), (2560, 64, 1536), (6912, 32, 4096), (6912, 16, 4160)]
+
+
+@pytest.mark.parametrize("K,N,S", SHAPES)
+def test_generator_equals_oracle(K, N, S):
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    Wo, po, no = oracle.generate(K, N, S)
+    assert (W == Wo).all() and (pos == po).all() and (neg == no).all()
+    p2, n2 = sp.lists_from_dense(W, S)
+    assert (p2 == pos).all() and (n2 == neg).all()
+
+
+def test_make_x_equals_oracle():
+    for seed, M, K in ((0xC0FFEE ^ 1, 1, 6912), (0xC0FFEE ^ 4, 4, 512), (7, 3, 64)):
+        assert (sp.make_x_i8(seed, M, K) == oracle.make_x_i8(seed, M, K)).all()
+
+
+@pytest.mark.parametrize("bad", [
+    dict(K=100, N=16, S=32), dict(K=64, N=20, S=32), dict(K=65536, N=16, S=32),
+    dict(K=64, N=16, S=31), dict(K=64, N=16, S=64), dict(K=0, N=16, S=0),
+])
+def test_shape_rules_of_init_ctx(bad):
+    # main.cu:85-91
+    with pytest.raises(sp.SptmmError) as e:
+        sp.generate_ternary(bad["K"], bad["N"], bad["S"])
+    assert e.value.code == -1
+
+
+@pytest.mark.parametrize("split", [8, 16, 32, 64, 128, 256])
+@pytest.mark.parametrize("K,N,S", [(2560, 64, 1536), (6912, 32, 4096), (6912, 16, 4160), (4096, 16, 3584)])
+def test_u16_stream_is_a_permutation_and_round_trips(K, N, S, split):
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    if (S // 2) % split:
+        with pytest.raises(sp.SptmmError):
+            sp.pack_u16(pos, neg, K, split)
+        return
+    pk = sp.pack_u16(pos, neg, K, split)
+    assert pk.nbytes == 2 * S * N  # exactly the algorithmic bytes: no padding
+    p2, n2 = sp.unpack_u16(pk, K, N, S, split)
+    assert (p2 == pos).all() and (n2 == neg).all()
+    allidx = np.sort(np.concatenate([pos.ravel(), neg.ravel()]))
+    assert (np.sort(pk.view(np.uint16)) == allidx).all()
+
+
+def test_u16_stream_offsets_closed_form():
+    # split 32, n_lane = 65 (S/2 = 2080): 8 full rounds + one 2-byte tail round
+    K, N, S, split = 6912, 16, 4160, 32
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    pk = sp.pack_u16(pos, neg, K, split).view(np.uint16)
+    n_lane = (S // 2) // split
+    task_words = 128 * n_lane
+    for c in (0, 1, 7, 15):
+        for i in (0, 31, 32, 255, 256, 2047, 2048, 2079):
+            lane = (c % 2) * 32 + i % split
+            slot = i // split
+            task = c // 2
+            if slot < 64:
+                off = (slot // 8) * 1024 + lane * 8 + slot % 8
+                offn = off + 512
+            else:
+                off = 8 * 1024 + lane
+                offn = off + 64
+            assert pk[task * task_words + off] == pos[c, i]
+            assert pk[task * task_words + offn] == neg[c, i]
+
+
+@pytest.mark.parametrize("split", [8, 16, 32, 64])
+@pytest.mark.parametrize("K,N,S", [(2560, 64, 1536), (6912, 32, 4096), (6912, 16, 4160), (6912, 16, 64)])
+def test_delta_stream_round_trips(K, N, S, split):
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    if (S // 2) % split:
+        return
+    bits = sp.delta_bits(pos, neg, split)
+    n_lane = (S // 2) // split
+    gaps_fit = True
+    for lst in (pos, neg):
+        runs = lst.reshape(N, split, n_lane).astype(int)
+        gaps_fit &= bool((np.diff(runs, axis=2) <= 255).all())
+    assert bits == (8 if gaps_fit else 16)
+    pk, b = sp.pack_delta(pos, neg, K, split)
+    assert b == bits and pk.nbytes == N // (64 // split) * (256 + 128 * n_lane * bits // 8)
+    p2, n2 = sp.unpack_delta(pk, K, N, S, split, bits)
+    assert (p2 == pos).all() and (n2 == neg).all()
+    if bits == 8:  # the wider form must carry the same lists
+        pk16, _ = sp.pack_delta(pos, neg, K, split, bits=16)
+        p3, n3 = sp.unpack_delta(pk16, K, N, S, split, 16)
+        assert (p3 == pos).all() and (n3 == neg).all()
+
+
+def test_delta_8bit_refuses_wide_gaps():
+    K, N, S = 6912, 16, 64  # mean gap ~200: some gaps exceed a byte
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    assert sp.delta_bits(pos, neg, 8) == 16
+    with pytest.raises(sp.SptmmError):
+        sp.pack_delta(pos, neg, K, 8, bits=8)
+
+
+def test_delta_gaps_match_oracle_within_runs():
+    # inside a run the stored bytes are the reference's gaps (main.cu:376-394)
+    K, N, S, split = 2560, 16, 1536, 32
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    d_ref, wrapped = oracle.delta8(pos)
+    assert wrapped == 0
+    pk, bits = sp.pack_delta(pos, neg, K, split)
+    assert bits == 8
+    n_lane = (S // 2) // split  # 24 = one 16-byte round + one 8-byte round
+    task_bytes = 256 + 128 * n_lane
+    for c in (0, 3, 15):
+        for v in (0, 5, 31):
+            lane = (c % 2) * 32 + v
+            t = pk[(c // 2) * task_bytes:(c // 2 + 1) * task_bytes]
+            restart = t[:256].view(np.uint16)[lane]
+            assert restart == pos[c, v * n_lane]
+            got = np.concatenate([t[256 + lane * 16: 256 + lane * 16 + 16],
+                                  t[256 + 2048 + lane * 8: 256 + 2048 + lane * 8 + 8]])
+            want = d_ref[c, v * n_lane:(v + 1) * n_lane].copy()
+            want[0] = 0
+            assert (got == want).all()
+
+
+def test_i2s_word_and_stream():
+    w = np.zeros(16, np.int8)
+    w[0], w[2] = 1, -1
+    assert sp.i2s_pack_word(w) == 0xAAA9AAAB == oracle.i2s_pack_word(w)
+    rng = np.random.default_rng(0)
+    for _ in range(50):
+        w = rng.integers(-1, 2, 16).astype(np.int8)
+        word = sp.i2s_pack_word(w)
+        assert word == oracle.i2s_pack_word(w)
+        assert (sp.i2s_decode_word(word) == w).all() and (oracle.i2s_decode_word(word) == w).all()
+    for K, N, S in ((512, 32, 300), (2560, 16, 1536), (6912, 16, 4096), (304, 16, 100)):
+        W, _, _ = sp.generate_ternary(K, N, S, dense=True)
+        pk = sp.pack_i2s(W)
+        Kp = (K + 255) // 256 * 256
+        assert pk.nbytes == N * Kp // 4
+        assert (sp.unpack_i2s(pk, K, N) == W).all()
+        # same multiset of words as the oracle's plain order (plus all-zero-weight pad words)
+        words = np.sort(pk.view(np.uint32))
+        ref = np.sort(np.concatenate([oracle.i2s_pack(W).ravel(),
+                                      np.full(N * (Kp - K) // 16, 0xAAAAAAAA, np.uint32)]))
+        assert (words == ref).all()
+
+
+def test_i2s_rejects_non_ternary():
+    W = np.zeros((16, 64), np.int8)
+    W[3, 5] = 2
+    with pytest.raises(sp.SptmmError):
+        sp.pack_i2s(W)

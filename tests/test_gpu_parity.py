@@ -1,0 +1,336 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
+
+Integer paths must be bit-exact.  Floating-point activation variants (fp16 /
+fp32 inputs, fp32 sums) must satisfy
+    max |got - ref| <= 1e-3 * max(|ref|, sqrt(S))          per element,
+with ref the float64 gather-sum (sqrt(S) is the scale of a sum of S unit-variance
+terms; it keeps the relative bound meaningful where the sum cancels to ~0).
+"""
+import hashlib
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import oracle
+import sptmm_amd as sp
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+_CACHE = {}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def device():
+    info = sp.device_init(0)
+    print("device:", info, flush=True)
+    return info
+
+
+def matrix(K, N, S, dense=False):
+    key = (K, N, S)
+    if key not in _CACHE or (dense and _CACHE[key][0] is None):
+        _CACHE.clear()  # keep host memory bounded
+        W, pos, neg = sp.generate_ternary(K, N, S, dense=dense)
+        Wo, po, no = oracle.generate(K, N, S, dense=False)
+        assert (pos == po).all() and (neg == no).all()
+        _CACHE[key] = (W, pos, neg)
+    return _CACHE[key]
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def x_i8(seed, M, K):
+    return oracle.make_x_i8(seed, M, K)
+
+
+def check_fp(got, ref, S):
+    scale = np.maximum(np.abs(ref), np.sqrt(S))
+    err = np.abs(got.astype(np.float64) - ref) / scale
+    assert err.max() <= REL_TOL, "max rel err %.3e" % err.max()
+
+
+# ------------------------------------------------------------------ u16 lists
+@pytest.mark.parametrize("split", [8, 16, 32, 64, 128, 256])
+@pytest.mark.parametrize("M", [1, 4])
+def test_u16_headline_shape_bit_exact(split, M, golden_dir):
+    K, N, S = 6912, 2560, 4096
+    say("u16 cfg0/1", K, N, S, "split", split, "M", M)
+    _, pos, neg = matrix(K, N, S)
+    X = x_i8(0xC0FFEE ^ M, M, K)
+    want = oracle.sptmm_i8_mt(X, pos, neg, 8)
+    w = sp.Weights.upload_u16(pos, neg, K, split)
+    assert w.nbytes == 2 * S * N
+    got = w.matmul(X)
+    w.free()
+    assert got.dtype == np.int32 and (got == want).all()
+    kats = json.load(open(os.path.join(golden_dir, "generator_kats.json")))
+    e = [m for m in kats["matrices"] if (m["K"], m["N"], m["S"]) == (K, N, S)][0]
+    o = [o for o in e["outputs"] if o["M"] == M][0]
+    assert hashlib.sha256(got.tobytes()).hexdigest() == o["sha256_C"]
+
+
+@pytest.mark.parametrize("M", [2, 3, 5, 7, 8, 9, 16])
+def test_u16_row_counts(M):
+    K, N, S = 6912, 256, 4096
+    say("u16 rows", M)
+    _, pos, neg = matrix(K, N, S)
+    X = x_i8(100 + M, M, K)
+    want = oracle.sptmm_i8_mt(X, pos, neg, 8)
+    for split in (32, 128):
+        w = sp.Weights.upload_u16(pos, neg, K, split)
+        got = w.matmul(X)
+        w.free()
+        assert (got == want).all(), split
+
+
+@pytest.mark.parametrize("K,N,S,splits", [
+    (64, 16, 32, (8, 16)),               # one or two entries per lane: tails only
+    (512, 48, 256, (8, 16, 32, 64, 128)),
+    (6912, 64, 4160, (8, 16, 32)),       # S/2 = 2080 = 32*65: ragged tail rounds
+    (2560, 640, 1536, (8, 16, 32, 64, 256)),
+    (4096, 32, 3584, (256,)),            # n_lane = 7: 8+4+2-byte tail rounds
+])
+def test_u16_ragged_and_small_shapes(K, N, S, splits):
+    _, pos, neg = matrix(K, N, S)
+    for M in (1, 4, 6):
+        X = x_i8(K + M, M, K)
+        want = oracle.sptmm_i8_mt(X, pos, neg, 4)
+        for split in splits:
+            say("u16 ragged", K, N, S, "split", split, "M", M)
+            w = sp.Weights.upload_u16(pos, neg, K, split)
+            got = w.matmul(X)
+            w.free()
+            assert (got == want).all(), (split, M)
+
+
+def test_u16_special_inputs():
+    K, N, S = 2560, 640, 1536
+    W, pos, neg = matrix(K, N, S, dense=True)
+    w = sp.Weights.upload_u16(pos, neg, K, 32)
+    say("u16 ones")
+    assert (w.matmul(np.ones((1, K), np.int8)) == 0).all()            # balanced signs
+    assert (w.matmul(np.full((2, K), -127, np.int8)) == 0).all()
+    for k in (0, 1, 1279, K - 1):
+        e = np.zeros((1, K), np.int8)
+        e[0, k] = 1
+        say("u16 unit", k)
+        assert (w.matmul(e)[0] == W[:, k]).all()                      # unit vector picks row k of W
+    X = np.full((1, K), 127, np.int8)
+    X[0, ::2] = -127
+    assert (w.matmul(X) == oracle.sptmm_i8(X, pos, neg)).all()        # extreme magnitudes
+    w.free()
+
+
+def test_linearity_and_split_invariance_full_size():
+    K, N, S = 6912, 2560, 4096
+    _, pos, neg = matrix(K, N, S)
+    rng = np.random.default_rng(11)
+    X1 = rng.integers(-60, 61, (4, K), dtype=np.int8)
+    X2 = rng.integers(-60, 61, (4, K), dtype=np.int8)
+    outs = []
+    for split in (8, 32, 64, 256):
+        say("linearity split", split)
+        w = sp.Weights.upload_u16(pos, neg, K, split)
+        a, b, ab = w.matmul(X1), w.matmul(X2), w.matmul((X1 + X2).astype(np.int8))
+        w.free()
+        assert (a + b == ab).all()
+        outs.append(ab)
+    for o in outs[1:]:
+        assert (o == outs[0]).all()
+
+
+# ---------------------------------------------------------------- gap streams
+@pytest.mark.parametrize("split", [8, 16, 32, 64])
+def test_delta_headline_shape_int8_bit_exact(split):
+    K, N, S = 6912, 2560, 4096
+    say("delta i8 split", split)
+    _, pos, neg = matrix(K, N, S)
+    w = sp.Weights.upload_delta(pos, neg, K, split)
+    assert w.info["delta_bits"] == 8
+    for M in (1, 4):
+        X = x_i8(0xC0FFEE ^ M, M, K)
+        assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), M
+    w.free()
+
+
+def test_delta_matches_reference_layout_walk():
+    # the oracle's walk of the reference's own div256 byte layout (main.cu:644-675)
+    K, N, S = 6912, 64, 4096
+    _, pos, neg = matrix(K, N, S)
+    dp, wp = oracle.delta8(pos)
+    dn, wn = oracle.delta8(neg)
+    assert wp == 0 and wn == 0
+    X = x_i8(77, 2, K)
+    want = oracle.sptmm_delta_i8(X, oracle.delta_div256(dp), oracle.delta_div256(dn), N, S // 2)
+    say("delta vs div256 walk")
+    w = sp.Weights.upload_delta(pos, neg, K, 32)
+    got = w.matmul(X)
+    w.free()
+    assert (got == want).all()
+
+
+def test_delta_fp16_config2():
+    K, N, S = 6912, 2560, 4096
+    _, pos, neg = matrix(K, N, S)
+    X = oracle.make_x_normal(2, 1, K, np.float16)
+    ref = oracle.sptmm_f64(X, pos, neg)
+    say("delta fp16 cfg2")
+    w = sp.Weights.upload_delta(pos, neg, K, 32)
+    got = w.matmul(X)
+    assert got.dtype == np.float32
+    check_fp(got, ref, S)
+    X4 = oracle.make_x_normal(3, 4, K, np.float16)
+    check_fp(w.matmul(X4), oracle.sptmm_f64(X4, pos, neg), S)
+    w.free()
+
+
+@pytest.mark.parametrize("K,N,S,splits", [
+    (6912, 32, 64, (8, 16, 32)),         # sparse: gaps above 255 -> 16-bit stream
+    (6912, 16, 256, (8, 64)),
+    (6912, 64, 4160, (8, 16, 32)),       # ragged: 65 / 130 / 260 gaps per lane
+    (2560, 640, 1536, (8, 16, 32, 64)),
+    (512, 48, 256, (8, 16, 32, 64)),
+    (64, 16, 32, (8, 16)),
+])
+def test_delta_ragged_sparse_and_16bit(K, N, S, splits):
+    _, pos, neg = matrix(K, N, S)
+    for split in splits:
+        w = sp.Weights.upload_delta(pos, neg, K, split)
+        bits = w.info["delta_bits"]
+        assert bits == sp.delta_bits(pos, neg, split)
+        for M in (1, 4, 5):
+            say("delta", K, N, S, "split", split, "bits", bits, "M", M)
+            X = x_i8(S + M, M, K)
+            assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 4)).all(), (split, M)
+        Xh = oracle.make_x_normal(split, 2, K, np.float16)
+        check_fp(w.matmul(Xh), oracle.sptmm_f64(Xh, pos, neg), S)
+        w.free()
+
+
+# ----------------------------------------------------- floating-point variants
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("M", [1, 3, 4])
+def test_u16_float_activations(dtype, M):
+    K, N, S = 6912, 2560, 4096
+    _, pos, neg = matrix(K, N, S)
+    X = oracle.make_x_normal(40 + M, M, K, dtype)
+    ref = oracle.sptmm_f64(X, pos, neg)
+    for split in (32, 128):
+        say("u16 float", dtype.__name__, "M", M, "split", split)
+        w = sp.Weights.upload_u16(pos, neg, K, split)
+        got = w.matmul(X)
+        w.free()
+        check_fp(got, ref, S)
+
+
+# ------------------------------------------------------------------------ i2s
+@pytest.mark.parametrize("K,N,S", [(6912, 2560, 4096), (2560, 2560, 1536), (2560, 640, 1536),
+                                   (2560, 6912, 1536), (304, 32, 100), (512, 48, 256), (64, 16, 32)])
+def test_i2s_bit_exact(K, N, S):
+    W, pos, neg = matrix(K, N, S, dense=True)
+    w = sp.Weights.upload_i2s(W)
+    assert w.nbytes == N * ((K + 255) // 256 * 256) // 4
+    for M in (1, 2, 4, 5, 8, 11):
+        say("i2s", K, N, S, "M", M)
+        X = x_i8(K ^ M, M, K)
+        assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), M
+    w.free()
+
+
+def test_i2s_matches_oracle_i2s_and_dense():
+    K, N, S = 512, 48, 256
+    W, pos, neg = matrix(K, N, S, dense=True)
+    X = x_i8(9, 3, K)
+    w = sp.Weights.upload_i2s(W)
+    got = w.matmul(X)
+    w.free()
+    assert (got == oracle.i2s_gemv(X, oracle.i2s_pack(W))).all()
+    assert (got == oracle.dense_i8(X, W)).all()
+
+
+# --------------------------------------------------------- benchmark configs 3, 4
+LAYER = [("q/o", 2560, 2560, 1536), ("k/v", 2560, 640, 1536), ("gate/up", 2560, 6912, 1536),
+         ("down", 6912, 2560, 4160)]
+
+
+@pytest.mark.parametrize("name,K,N,S", LAYER)
+def test_decoder_layer_shapes_all_formats(name, K, N, S):
+    W, pos, neg = matrix(K, N, S, dense=True)
+    ws = [sp.Weights.upload_u16(pos, neg, K, 32), sp.Weights.upload_delta(pos, neg, K, 32), sp.Weights.upload_i2s(W)]
+    for M in (1, 4):
+        X = x_i8(1000 + M, M, K)
+        want = oracle.sptmm_i8_mt(X, pos, neg, 8)
+        for w in ws:
+            say("layer", name, "kind", w.info["kind"], "M", M)
+            assert (w.matmul(X) == want).all(), (name, w.info, M)
+    for w in ws:
+        w.free()
+
+
+def test_large_layer_config4_three_encodings():
+    K, N, S = 13824, 5120, 8320
+    W, pos, neg = matrix(K, N, S, dense=True)
+    ws = [sp.Weights.upload_u16(pos, neg, K, 32), sp.Weights.upload_u16(pos, neg, K, 64),
+          sp.Weights.upload_delta(pos, neg, K, 32), sp.Weights.upload_i2s(W)]
+    assert ws[0].nbytes == 2 * S * N and ws[3].nbytes == K * N // 4
+    for M in (1, 8, 16):
+        X = x_i8(4000 + M, M, K)
+        want = oracle.sptmm_i8_mt(X, pos, neg, 8)
+        for w in ws:
+            say("cfg4 kind", w.info["kind"], "split", w.info["split_k"], "M", M)
+            assert (w.matmul(X) == want).all(), (w.info, M)
+    for w in ws:
+        w.free()
+
+
+# ------------------------------------------------------------- boundary behaviour
+def test_argument_errors_are_status_codes():
+    K, N, S = 512, 48, 256
+    _, pos, neg = matrix(K, N, S)
+    with pytest.raises(sp.SptmmError) as e:
+        sp.Weights.upload_u16(pos, neg, K, 12)
+    assert e.value.code == -1 and "split" in str(e.value).lower()
+    with pytest.raises(sp.SptmmError):
+        sp.Weights.upload_delta(pos, neg, K, 128)
+    w = sp.Weights.upload_delta(pos, neg, K, 32)
+    xb = sp.DeviceBuffer(K)
+    cb = sp.DeviceBuffer(4 * N)
+    with pytest.raises(sp.SptmmError):
+        w.gemv_i8(xb, 0, cb)
+    W = np.zeros((N, K), np.int8)
+    wi = sp.Weights.upload_i2s(W)
+    with pytest.raises(sp.SptmmError) as e:
+        wi.gemv_f16(xb, 1, cb)
+    assert e.value.code == -2
+    for o in (w, wi, xb, cb):
+        o.free()
+
+
+def test_streams_and_clone():
+    K, N, S = 2560, 640, 1536
+    _, pos, neg = matrix(K, N, S)
+    X = x_i8(5, 1, K)
+    want = oracle.sptmm_i8(X, pos, neg)
+    w = sp.Weights.upload_u16(pos, neg, K, 32)
+    w2 = w.clone()
+    st = sp.Stream()
+    xb = sp.DeviceBuffer.from_numpy(X)
+    cb = sp.DeviceBuffer(4 * N)
+    ev0, ev1 = sp.Event(), sp.Event()
+    ev0.record(st)
+    for _ in range(10):
+        w2.gemv_i8(xb, 1, cb, st)
+    ev1.record(st)
+    ev1.sync()
+    assert ev0.elapsed_us(ev1) > 0
+    assert (cb.to_numpy(np.int32, (1, N)) == want).all()
+    for o in (w, w2, xb, cb):
+        o.free()
+    st.destroy()
