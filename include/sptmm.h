@@ -159,9 +159,11 @@ int sptmm_event_elapsed_us(void *start, void *stop, double *us);
  * cache).  act: 0 int8, 1 fp16, 2 fp32.  mode: 0 = back-to-back launches on one
  * stream between two events; 1 = stream synchronize after every launch, as the
  * reference does (main.cu:1456); 2 = one rotation captured into a HIP graph and
- * replayed.  Reports mean microseconds per launch. */
+ * replayed.  `stream` must come from sptmm_stream_create; the call returns after
+ * the stream has drained.  Reports mean microseconds per launch, taken from two
+ * events recorded on that stream. */
 int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X_dev, int M, void *C_dev,
-                       int iters, int mode, double *us_per_call);
+                       int iters, int mode, void *stream, double *us_per_call);
 /* Reads `bytes` of a scratch buffer and writes them back (a plain copy kernel):
  * evicts cached weight streams between cold-read timings and calibrates the
  * traffic counters. */

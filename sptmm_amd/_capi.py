@@ -81,7 +81,7 @@ def lib() -> C.CDLL:
         L.sptmm_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.sptmm_memset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
         L.sptmm_measure_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
-                                         C.c_int, C.POINTER(C.c_double)]
+                                         C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         L.sptmm_copy_kernel.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         L.sptmm_make_x_i8.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p]
         for n in ("sptmm_stream_create", "sptmm_event_create"):
@@ -277,11 +277,19 @@ class Event:
             self.handle = C.c_void_p()
 
 
-def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuffer", iters: int, mode: int = 0) -> float:
+def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuffer", iters: int, mode: int = 0,
+                 stream: "Stream | None" = None) -> float:
     """Mean microseconds per launch over `iters` launches rotating over `weights` (see sptmm_measure_gemv)."""
     arr = (C.c_void_p * len(weights))(*[w.handle for w in weights])
     us = C.c_double()
-    _ck(lib().sptmm_measure_gemv(arr, len(weights), act, X.ptr, M, Cout.ptr, iters, mode, C.byref(us)))
+    own = stream is None
+    if own:
+        stream = Stream()
+    try:
+        _ck(lib().sptmm_measure_gemv(arr, len(weights), act, X.ptr, M, Cout.ptr, iters, mode, stream.handle, C.byref(us)))
+    finally:
+        if own:
+            stream.destroy()
     return us.value
 
 

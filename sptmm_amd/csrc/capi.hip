@@ -101,6 +101,7 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.G = w->geo.G;
     a.W = w->geo.W;
     a.delta_bits = w->info.delta_bits;
+    a.index_shift = w->info.kind == SPTMM_KIND_U16 ? u16_index_shift(w->info.K) : 0;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
     switch (w->info.kind) {
@@ -313,11 +314,12 @@ int sptmm_event_elapsed_us(void *a, void *b, double *us)
     return SPTMM_OK;
 }
 int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters,
-                       int mode, double *us_per_call)
+                       int mode, void *stream, double *us_per_call)
 {
     if (!ws || n_ws < 1 || !X || !C || iters < 1 || !us_per_call) return fail(SPTMM_ERR_INVALID, "bad argument");
     if (act < ACT_I8 || act > ACT_F32 || mode < 0 || mode > 2) return fail(SPTMM_ERR_INVALID, "bad act or mode");
-    hipStream_t st = nullptr;
+    if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_measure_gemv needs a stream made by sptmm_stream_create");
+    hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -332,7 +334,6 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
             goto done;                     \
         }                                  \
     } while (0)
-    M_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
     M_TRY(hipEventCreate(&e0));
     M_TRY(hipEventCreate(&e1));
     if (mode == 2) {
@@ -370,10 +371,7 @@ done:
     if (graph) (void)hipGraphDestroy(graph);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
-    if (st) {
-        (void)hipStreamSynchronize(st);
-        (void)hipStreamDestroy(st);
-    }
+    (void)hipStreamSynchronize(st);
     return rc;
 }
 

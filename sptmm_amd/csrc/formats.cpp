@@ -3,6 +3,7 @@
 // machine.  The streams are laid out for 64-lane wavefronts: every per-lane
 // load of a wavefront touches one contiguous, naturally aligned block.
 #include <algorithm>
+#include <array>
 #include <cstdio>
 #include <cstring>
 #include <thread>
@@ -190,6 +191,8 @@ int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X)
 }
 
 // ------------------------------------------------------------------ u16 stream
+// Stored fields are row indices, multiplied by 4 (the byte offset of the row's
+// 4-byte LDS slot) whenever 4*K still fits 16 bits.
 size_t sptmm_pack_u16_bytes(int N, int S, int split_k)
 {
     Geometry g;
@@ -197,41 +200,168 @@ size_t sptmm_pack_u16_bytes(int N, int S, int split_k)
     return (size_t)g.tasks * 256 * g.n_lane;
 }
 
-static int u16_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int K, int N, int S, int split_k)
+}  // extern "C"
+
+namespace sptmm {
+
+// One scheduling domain = the 32 lanes of a half-wavefront, which the LDS
+// serves in one pass when they hit 32 different banks (bank = row index mod 32
+// in every tile layout).  `owners` columns share the domain, each with `lanes`
+// lanes (owners*lanes == 32) and lanes*n entries.  Entries of a slot are chosen
+// bank by bank, fullest bank first, so that conflicts only appear once some
+// bank has run dry, and land in as few slots as possible.
+struct Domain {
+    int owners, lanes, n;
+    std::vector<std::vector<uint16_t>> entries;          // per owner
+    std::vector<std::vector<uint16_t>> cell;             // per owner: [slot][lane] -> index
+};
+
+void schedule(Domain &d)
+{
+    const int no = d.owners, Lo = d.lanes, n = d.n;
+    std::vector<std::array<std::vector<uint16_t>, 32>> pool(no);
+    for (int o = 0; o < no; ++o)
+        for (uint16_t k : d.entries[o]) pool[o][k & 31].push_back(k);
+    d.cell.assign(no, std::vector<uint16_t>((size_t)n * Lo));
+    std::vector<int> need(no);
+    std::vector<std::vector<uint16_t>> pick(no);
+    for (int slot = 0; slot < n; ++slot) {
+        int open = 0;
+        for (int o = 0; o < no; ++o) {
+            need[o] = Lo;
+            pick[o].clear();
+            open += Lo;
+        }
+        while (open > 0) {  // one sweep = one more entry allowed per bank
+            int order[32], total[32];
+            for (int b = 0; b < 32; ++b) {
+                order[b] = b;
+                total[b] = 0;
+                for (int o = 0; o < no; ++o) total[b] += (int)pool[o][b].size();
+            }
+            std::sort(order, order + 32, [&](int x, int y) { return total[x] != total[y] ? total[x] > total[y] : x < y; });
+            for (int i = 0; i < 32 && open > 0; ++i) {
+                const int b = order[i];
+                int who = -1;
+                for (int o = 0; o < no; ++o)
+                    if (need[o] > 0 && !pool[o][b].empty() && (who < 0 || pool[o][b].size() > pool[who][b].size())) who = o;
+                if (who < 0) continue;
+                pick[who].push_back(pool[who][b].back());
+                pool[who][b].pop_back();
+                --need[who];
+                --open;
+            }
+        }
+        for (int o = 0; o < no; ++o) {
+            std::sort(pick[o].begin(), pick[o].end(), [](uint16_t x, uint16_t y) { return (x & 31) != (y & 31) ? (x & 31) < (y & 31) : x < y; });
+            for (int l = 0; l < Lo; ++l) d.cell[o][(size_t)slot * Lo + l] = pick[o][l];
+        }
+    }
+}
+
+int u16_index_shift(int K) { return 4 * K <= 65535 ? 2 : 0; }
+
+// Cells of the stream that belong to (column c, sign): calls f(task, lane, slot, i) for i = 0..half-1
+// in a fixed enumeration order: part-major, then half-wavefront, then slot, then lane.
+template <class F>
+void for_cells(const Geometry &g, int c, F f)
+{
+    int i = 0;
+    if (g.L == 64) {
+        for (int part = 0; part < g.W; ++part)
+            for (int h = 0; h < 2; ++h)
+                for (int slot = 0; slot < g.n_lane; ++slot)
+                    for (int l = 0; l < 32; ++l) f(c * g.W + part, 32 * h + l, slot, i++);
+    } else {
+        const int task = c / g.G, l0 = (c % g.G) * g.L;
+        for (int slot = 0; slot < g.n_lane; ++slot)
+            for (int l = 0; l < g.L; ++l) f(task, l0 + l, slot, i++);
+    }
+}
+
+}  // namespace sptmm
+
+extern "C" {
+
+int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out)
 {
     if (int rc = check_shape(K, N, S)) return rc;
     Geometry g;
     if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
-    if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (!out || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    for (size_t i = 0, n = (size_t)N * g.half; i < n; ++i)
+        if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
+    const int sh = u16_index_shift(K);
     const size_t task_bytes = (size_t)256 * g.n_lane;
-    uint8_t *base = (uint8_t *)packed;
-    parallel_columns(N, [&](int c) {
+    uint8_t *base = (uint8_t *)out;
+    auto put = [&](int task, int lane, int slot, int sign, uint16_t k) {
+        *(uint16_t *)(base + task * task_bytes + slot_offset(g.n_lane, 2, sign, lane, slot)) = (uint16_t)(k << sh);
+    };
+    // groups of columns that share half-wavefronts: one column when L >= 32, else 32/L columns
+    const int group = g.L >= 32 ? 1 : 32 / g.L;
+    parallel_columns(N / group, [&](int gi) {
         for (int sign = 0; sign < 2; ++sign) {
-            uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
-            for (int i = 0; i < g.half; ++i) {
-                Place p = place(g, c, i, false);
-                uint16_t *cell = (uint16_t *)(base + p.task * task_bytes + slot_offset(g.n_lane, 2, sign, p.lane, p.slot));
-                if (pack)
-                    *cell = lst[i];
-                else
-                    lst[i] = *cell;
+            const uint16_t *lists = sign ? neg : pos;
+            if (g.L == 64) {
+                // deal the column's entries, bank by bank, round-robin over its 2*W half-wavefronts
+                const int c = gi, nd = 2 * g.W;
+                std::vector<uint16_t> e(lists + (size_t)c * g.half, lists + (size_t)(c + 1) * g.half);
+                std::stable_sort(e.begin(), e.end(), [](uint16_t x, uint16_t y) { return (x & 31) < (y & 31); });
+                std::vector<Domain> dom(nd);
+                for (int d = 0; d < nd; ++d) {
+                    dom[d].owners = 1;
+                    dom[d].lanes = 32;
+                    dom[d].n = g.n_lane;
+                    dom[d].entries.resize(1);
+                }
+                for (int i = 0; i < g.half; ++i) dom[i % nd].entries[0].push_back(e[i]);
+                for (int d = 0; d < nd; ++d) {
+                    schedule(dom[d]);
+                    for (int slot = 0; slot < g.n_lane; ++slot)
+                        for (int l = 0; l < 32; ++l)
+                            put(c * g.W + d / 2, 32 * (d % 2) + l, slot, sign, dom[d].cell[0][(size_t)slot * 32 + l]);
+                }
+            } else {
+                Domain d;
+                d.owners = group;
+                d.lanes = g.L >= 32 ? 32 : g.L;
+                d.n = g.n_lane;
+                d.entries.resize(group);
+                for (int o = 0; o < group; ++o) {
+                    const int c = gi * group + o;
+                    d.entries[o].assign(lists + (size_t)c * g.half, lists + (size_t)(c + 1) * g.half);
+                }
+                schedule(d);
+                for (int o = 0; o < group; ++o) {
+                    const int c = gi * group + o, task = c / g.G, l0 = (c % g.G) * g.L;
+                    for (int slot = 0; slot < g.n_lane; ++slot)
+                        for (int l = 0; l < d.lanes; ++l) put(task, l0 + l, slot, sign, d.cell[o][(size_t)slot * d.lanes + l]);
+                }
             }
         }
     });
     return SPTMM_OK;
 }
 
-int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out)
-{
-    if (pos && neg)
-        for (size_t i = 0, n = (size_t)N * (S / 2); i < n; ++i)
-            if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
-    return u16_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k);
-}
-
 int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg)
 {
-    return u16_walk(false, (void *)packed, pos, neg, K, N, S, split_k);
+    if (int rc = check_shape(K, N, S)) return rc;
+    Geometry g;
+    if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
+    if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    const int sh = u16_index_shift(K);
+    const size_t task_bytes = (size_t)256 * g.n_lane;
+    const uint8_t *base = (const uint8_t *)packed;
+    parallel_columns(N, [&](int c) {
+        for (int sign = 0; sign < 2; ++sign) {
+            uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
+            for_cells(g, c, [&](int task, int lane, int slot, int i) {
+                lst[i] = (uint16_t)(*(const uint16_t *)(base + task * task_bytes + slot_offset(g.n_lane, 2, sign, lane, slot)) >> sh);
+            });
+            std::sort(lst, lst + g.half);
+        }
+    });
+    return SPTMM_OK;
 }
 
 // ---------------------------------------------------------------- gap streams

@@ -32,6 +32,9 @@ int make_geometry(int N, int S, int split_k, int max_split, Geometry *g);
 // round each of 8, 4, 2 and (esz==1) 1 bytes per lane.
 size_t slot_offset(int n_lane, int esz, int sign, int lane, int j);
 
+// u16 stream fields are row indices shifted left by this many bits (2 when 4*K fits 16 bits).
+int u16_index_shift(int K);
+
 // i2s tiling: 16 columns x 4 lanes per wave-load, 16 bytes (64 weights) per lane.
 inline int i2s_padded_k(int K) { return (K + 255) / 256 * 256; }
 
@@ -45,6 +48,7 @@ struct GemvArgs {
     void *C;            // device output, row-major [M][N]
     int M, K, N, half, split_k, n_lane, tasks, L, G, W;
     int delta_bits;
+    int index_shift;    // u16 stream: fields are row << index_shift
     int compute_units;
     int lds_limit;
 };
