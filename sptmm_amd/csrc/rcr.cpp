@@ -1,0 +1,359 @@
+// rcr -- bench driver with the command line of the reference benchmark
+// (main.cu:38-49 flags, main.cu:813-832 banner, one bare "ms per call" float per
+// selected method as at main.cu:1459/1845/1962), running on the C ABI of
+// libsptmm.so.  No HIP headers here.
+//
+//   ./rcr -row_split3_small 32 -M=1 -K=6912 -N=2560 -S=4096 -iter=100000
+//   ./rcr -row_split_delta2 32 -M=1 -K=6912 -N=2560 -S=4096 -iter=100000
+//   ./rcr -i2s -M=1 -K=6912 -N=2560 -S=4096 -iter=100000
+//
+// Unlike the reference, any shape that passes its own validity rules runs (there
+// is no table of compiled-in shapes), activations are seeded, and results are
+// checked: the three encodings of the same matrix must agree.
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <iostream>
+#include <string>
+#include <vector>
+
+#include "../../include/sptmm.h"
+
+namespace {
+
+struct Flags {
+    bool cu_blas = false, i2s = false, check = true, help = false;
+    uint64_t row_split3_small = 0, row_split_delta2 = 0;
+    uint64_t M = 32, K = 3072, N = 768, S = 256, L = 1;  // defaults of main.cu:43-47
+    uint32_t iter = 10;
+    // additions of this build
+    uint64_t cold = 0;      // rotate over this many device copies of the stream (0 = one copy, as the reference)
+    uint64_t seed = 0;      // activation seed (0 = 0xC0FFEE ^ M)
+    std::string act = "i8"; // i8 | f16 | f32
+};
+
+[[noreturn]] void strict_fail(const char *msg)
+{
+    // STRICT_ASSERT of macro.cuh:66
+    fprintf(stderr, "%s\n", msg);
+    abort();
+}
+
+#define CHECK_SPTMM(expr)                                                                          \
+    do {                                                                                           \
+        int rc_ = (expr);                                                                          \
+        if (rc_ == SPTMM_ERR_INVALID) strict_fail(sptmm_last_error());                             \
+        if (rc_ != SPTMM_OK) {                                                                     \
+            fprintf(stderr, "HIP error at %s:%d code=%d \"%s\" (%s)\n", __FILE__, __LINE__, rc_,   \
+                    #expr, sptmm_last_error());                                                    \
+            exit(EXIT_FAILURE);                                                                    \
+        }                                                                                          \
+    } while (0)
+
+bool parse_bool(const std::string &v, bool *out)
+{
+    if (v == "true" || v == "1" || v == "t" || v == "yes" || v == "y") return *out = true, true;
+    if (v == "false" || v == "0" || v == "f" || v == "no" || v == "n") return *out = false, true;
+    return false;
+}
+
+// gflags grammar as the reference's README uses it: one or two dashes, "-flag value" or
+// "-flag=value"; booleans also as "-flag" / "-noflag".  Unknown flag: message + exit 1.
+void parse(int argc, char **argv, Flags &f)
+{
+    struct Spec {
+        const char *name;
+        int kind;  // 0 bool, 1 u64, 2 u32, 3 string
+        void *dst;
+    } specs[] = {
+        {"cu_blas", 0, &f.cu_blas}, {"i2s", 0, &f.i2s}, {"check", 0, &f.check}, {"help", 0, &f.help},
+        {"row_split3_small", 1, &f.row_split3_small}, {"row_split_delta2", 1, &f.row_split_delta2},
+        {"M", 1, &f.M}, {"K", 1, &f.K}, {"N", 1, &f.N}, {"S", 1, &f.S}, {"L", 1, &f.L},
+        {"iter", 2, &f.iter}, {"cold", 1, &f.cold}, {"seed", 1, &f.seed}, {"act", 3, &f.act},
+    };
+    for (int i = 1; i < argc; ++i) {
+        std::string a = argv[i];
+        if (a == "--") break;
+        if (a.size() < 2 || a[0] != '-') {
+            fprintf(stderr, "ERROR: unexpected argument '%s'\n", a.c_str());
+            exit(1);
+        }
+        a = a.substr(a[1] == '-' ? 2 : 1);
+        std::string name = a, val;
+        bool has_val = false;
+        size_t eq = a.find('=');
+        if (eq != std::string::npos) {
+            name = a.substr(0, eq);
+            val = a.substr(eq + 1);
+            has_val = true;
+        }
+        Spec *sp = nullptr;
+        bool negated = false;
+        for (auto &s : specs)
+            if (name == s.name) sp = &s;
+        if (!sp && name.rfind("no", 0) == 0)
+            for (auto &s : specs)
+                if (s.kind == 0 && name.substr(2) == s.name) sp = &s, negated = true;
+        if (!sp) {
+            fprintf(stderr, "ERROR: unknown command line flag '%s'\n", name.c_str());
+            exit(1);
+        }
+        if (sp->kind == 0) {
+            bool b = !negated;
+            if (has_val && (negated || !parse_bool(val, &b))) {
+                fprintf(stderr, "ERROR: illegal value '%s' specified for bool flag '%s'\n", val.c_str(), sp->name);
+                exit(1);
+            }
+            *(bool *)sp->dst = b;
+            continue;
+        }
+        if (!has_val) {
+            if (i + 1 >= argc) {
+                fprintf(stderr, "ERROR: flag '%s' is missing its argument\n", sp->name);
+                exit(1);
+            }
+            val = argv[++i];
+        }
+        if (sp->kind == 3) {
+            *(std::string *)sp->dst = val;
+            continue;
+        }
+        char *end = nullptr;
+        unsigned long long v = strtoull(val.c_str(), &end, 0);
+        if (val.empty() || *end || val[0] == '-' || (sp->kind == 2 && v > 0xffffffffull)) {
+            fprintf(stderr, "ERROR: illegal value '%s' specified for %s flag '%s'\n", val.c_str(),
+                    sp->kind == 1 ? "uint64" : "uint32", sp->name);
+            exit(1);
+        }
+        if (sp->kind == 1)
+            *(uint64_t *)sp->dst = v;
+        else
+            *(uint32_t *)sp->dst = (uint32_t)v;
+    }
+}
+
+uint32_t xorshift32(uint32_t &s)
+{
+    s ^= s << 13;
+    s ^= s >> 17;
+    s ^= s << 5;
+    return s;
+}
+
+uint16_t float_to_half(float x)
+{
+    uint32_t b;
+    memcpy(&b, &x, 4);
+    uint32_t sign = (b >> 16) & 0x8000u;
+    int32_t e = (int32_t)((b >> 23) & 0xff) - 127 + 15;
+    uint32_t m = b & 0x7fffffu;
+    if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign;
+        m |= 0x800000u;
+        uint32_t shift = (uint32_t)(14 - e);
+        uint32_t h = m >> shift, rem = m & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (h & 1))) ++h;
+        return (uint16_t)(sign | h);
+    }
+    uint32_t h = ((uint32_t)e << 10) | (m >> 13), rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1))) ++h;
+    return (uint16_t)(sign | h);
+}
+
+// ~N(0,1) from the same xorshift stream (Box-Muller)
+void make_x_normal(uint32_t seed, size_t n, std::vector<float> &out)
+{
+    uint32_t st = seed ? seed : 1u;
+    out.resize(n);
+    for (size_t i = 0; i < n; i += 2) {
+        double u1 = (xorshift32(st) + 1.0) / 4294967297.0, u2 = xorshift32(st) / 4294967296.0;
+        double r = std::sqrt(-2.0 * std::log(u1));
+        out[i] = (float)(r * std::cos(6.283185307179586 * u2));
+        if (i + 1 < n) out[i + 1] = (float)(r * std::sin(6.283185307179586 * u2));
+    }
+}
+
+struct Method {
+    const char *label;
+    sptmm_weights *w;
+    std::vector<unsigned char> result;  // device output copied back (int32 or float)
+};
+
+}  // namespace
+
+int main(int argc, char **argv)
+{
+    Flags f;
+    parse(argc, argv, f);
+    if (f.help) {
+        printf("matrix multiply speed check\n"
+               "  -row_split3_small <splitK>  SpTMM over u16 index lists (8,16,32,64,128,256)\n"
+               "  -row_split_delta2 <splitK>  SpTMM-delta over 8/16-bit gap streams (8,16,32,64)\n"
+               "  -i2s                        2-bit packed dense-ternary baseline\n"
+               "  -cu_blas                    not available in this layout (aborts like the reference's rcr)\n"
+               "  -M -K -N -S -L -iter        shape, nonzeros per column, iterations\n"
+               "  -act i8|f16|f32  -seed <n>  -cold <copies>  -nocheck\n");
+        return 0;
+    }
+    const int M = (int)f.M, K = (int)f.K, N = (int)f.N, S = (int)f.S;
+    const int act = f.act == "i8" ? 0 : f.act == "f16" ? 1 : f.act == "f32" ? 2 : -1;
+    if (act < 0) strict_fail("act must be i8, f16 or f32");
+    if (f.M < 1 || f.M > (1u << 20)) strict_fail("M out of range");
+
+    // host side first (needs no GPU): shape rules of main.cu:85-91 and the seeded ternary matrix
+    const bool any = f.row_split3_small || f.row_split_delta2 || f.i2s;
+    std::vector<uint16_t> pos, neg;
+    std::vector<int8_t> dense;
+    if (any) {
+        pos.resize((size_t)N * (size_t)std::max(S / 2, 0));
+        neg.resize(pos.size());
+        if ((f.i2s || f.check) && K > 0 && N > 0) dense.resize((size_t)K * N);
+        CHECK_SPTMM(sptmm_generate_ternary(K, N, S, dense.empty() ? nullptr : dense.data(), pos.data(), neg.data()));
+        if (f.row_split3_small && !sptmm_pack_u16_bytes(N, S, (int)f.row_split3_small)) strict_fail("Wrong split size");
+        if (f.row_split_delta2 && !sptmm_pack_delta_bytes(N, S, (int)f.row_split_delta2, 8)) strict_fail("Wrong split size");
+    }
+
+    sptmm_devinfo dev;
+    CHECK_SPTMM(sptmm_device_init(0, &dev));
+
+    // activations (make_X, main.cu:784-797; seeded here)
+    const uint32_t seed = f.seed ? (uint32_t)f.seed : (0xC0FFEEu ^ (uint32_t)M);
+    const size_t xcount = (size_t)M * K, esz = act == 0 ? 1 : act == 1 ? 2 : 4;
+    std::vector<unsigned char> xhost(xcount * esz);
+    if (act == 0) {
+        CHECK_SPTMM(sptmm_make_x_i8(seed, xcount, (int8_t *)xhost.data()));
+    } else {
+        std::vector<float> xf;
+        make_x_normal(seed, xcount, xf);
+        if (act == 2)
+            memcpy(xhost.data(), xf.data(), xcount * 4);
+        else
+            for (size_t i = 0; i < xcount; ++i) ((uint16_t *)xhost.data())[i] = float_to_half(xf[i]);
+    }
+    void *x_d = nullptr, *c_d = nullptr, *stream = nullptr;
+    CHECK_SPTMM(sptmm_malloc(&x_d, xhost.size()));
+    CHECK_SPTMM(sptmm_memcpy_h2d(x_d, xhost.data(), xhost.size()));
+    std::cout << "make_X done" << std::endl;
+    CHECK_SPTMM(sptmm_malloc(&c_d, sizeof(int) * (size_t)M * N));
+    CHECK_SPTMM(sptmm_memset(c_d, 0, sizeof(int) * (size_t)M * N));
+    CHECK_SPTMM(sptmm_stream_create(&stream));
+
+    printf("Compiled on %s at %s\n", __DATE__, __TIME__);
+    std::cout << "Start: "
+              << "M=" << f.M << " K=" << f.K << " N=" << f.N << " ITER=" << f.iter << " S=" << f.S << " ("
+              << (100.0 - 100.0 * ((float)f.S / (float)f.K)) << "% Sparsity)"
+              << " L=" << f.L << " B=" << 8 << " X_MAJOR=ROW W_MAJOR=COL C_MAJOR=ROW" << std::endl;
+
+    if (f.cu_blas) strict_fail("Wrong layout");  // main.cu:843: the row/col/row build refuses cuBLAS
+
+    std::vector<Method> done;
+    auto run = [&](const char *label, sptmm_weights *w, bool timed) {
+        sptmm_winfo wi;
+        CHECK_SPTMM(sptmm_weights_info(w, &wi));
+        const int a = wi.kind == SPTMM_KIND_I2S ? 0 : act;
+        if (wi.kind == SPTMM_KIND_I2S && act != 0) strict_fail("i2s takes int8 activations");
+        // one checked call first
+        CHECK_SPTMM(sptmm_memset(c_d, 0xff, sizeof(int) * (size_t)M * N));
+        if (a == 0)
+            CHECK_SPTMM(sptmm_gemv_i8(w, (const int8_t *)x_d, M, (int32_t *)c_d, stream));
+        else if (a == 1)
+            CHECK_SPTMM(sptmm_gemv_f16(w, (const uint16_t *)x_d, M, (float *)c_d, stream));
+        else
+            CHECK_SPTMM(sptmm_gemv_f32(w, (const float *)x_d, M, (float *)c_d, stream));
+        CHECK_SPTMM(sptmm_stream_sync(stream));
+        Method m{label, w, std::vector<unsigned char>(sizeof(int) * (size_t)M * N)};
+        CHECK_SPTMM(sptmm_memcpy_d2h(m.result.data(), c_d, m.result.size()));
+        if (timed) {
+            const int iters = (int)std::max<uint32_t>(f.iter, 1);
+            double us_sync = 0, us_b2b = 0, us_cold = 0;
+            const sptmm_weights *one[1] = {w};
+            // reference protocol: launch + synchronize per iteration (main.cu:1456)
+            CHECK_SPTMM(sptmm_measure_gemv(one, 1, a, x_d, M, c_d, iters, 1, stream, &us_sync));
+            std::cout << (float)(us_sync / 1000.0) << std::endl;
+            const int warm = std::min(iters, 200);
+            CHECK_SPTMM(sptmm_measure_gemv(one, 1, a, x_d, M, c_d, warm, 0, stream, &us_b2b));
+            CHECK_SPTMM(sptmm_measure_gemv(one, 1, a, x_d, M, c_d, iters, 0, stream, &us_b2b));
+            const double bytes = (double)wi.stream_bytes + (double)M * K * esz + 4.0 * M * N;
+            printf("# %s: us/call sync_each=%.3f back_to_back=%.3f (%.1f GB/s, %.1f%% of %.0f)", label, us_sync, us_b2b,
+                   bytes / us_b2b / 1e3, bytes / us_b2b / 1e3 / dev.peak_hbm_gbps * 100.0, dev.peak_hbm_gbps);
+            if (f.cold > 1) {
+                std::vector<sptmm_weights *> copies{w};
+                for (uint64_t i = 1; i < f.cold; ++i) {
+                    sptmm_weights *c = nullptr;
+                    CHECK_SPTMM(sptmm_weights_clone(w, &c));
+                    copies.push_back(c);
+                }
+                std::vector<const sptmm_weights *> cc(copies.begin(), copies.end());
+                CHECK_SPTMM(sptmm_measure_gemv(cc.data(), (int)cc.size(), a, x_d, M, c_d, (int)cc.size() * 2, 0, stream, &us_cold));
+                CHECK_SPTMM(sptmm_measure_gemv(cc.data(), (int)cc.size(), a, x_d, M, c_d, iters, 0, stream, &us_cold));
+                printf(" cold[%d copies]=%.3f (%.1f GB/s, %.1f%%)", (int)cc.size(), us_cold, bytes / us_cold / 1e3,
+                       bytes / us_cold / 1e3 / dev.peak_hbm_gbps * 100.0);
+                for (size_t i = 1; i < copies.size(); ++i) sptmm_weights_free(copies[i]);
+            }
+            printf(" bytes=%.0f kind=%d split_k=%d delta_bits=%d\n", bytes, wi.kind, wi.split_k, wi.delta_bits);
+        }
+        done.push_back(std::move(m));
+    };
+
+    if (f.row_split3_small > 0) {
+        sptmm_weights *w = nullptr;
+        CHECK_SPTMM(sptmm_weights_upload_u16(pos.data(), neg.data(), K, N, S, (int)f.row_split3_small, &w));
+        run("sptmm", w, true);
+    }
+    if (f.row_split_delta2 > 0) {
+        sptmm_weights *w = nullptr;
+        CHECK_SPTMM(sptmm_weights_upload_delta(pos.data(), neg.data(), K, N, S, (int)f.row_split_delta2, &w));
+        run("sptmm-delta", w, true);
+    }
+    if (f.i2s) {
+        sptmm_weights *w = nullptr;
+        CHECK_SPTMM(sptmm_weights_upload_i2s(dense.data(), K, N, &w));
+        run("i2s", w, true);
+    }
+
+    int status = 0;
+    if (any && f.check) {
+        // the encodings are independent: make sure at least two of them have run, then compare all
+        if (done.size() < 2) {
+            sptmm_weights *w = nullptr;
+            if (act == 0 && !f.i2s) {
+                CHECK_SPTMM(sptmm_weights_upload_i2s(dense.data(), K, N, &w));
+                run("i2s(check)", w, false);
+            } else if (!f.row_split3_small && (S / 2) % 32 == 0) {
+                CHECK_SPTMM(sptmm_weights_upload_u16(pos.data(), neg.data(), K, N, S, 32, &w));
+                run("sptmm(check)", w, false);
+            } else if ((S / 2) % 8 == 0) {
+                CHECK_SPTMM(sptmm_weights_upload_delta(pos.data(), neg.data(), K, N, S, 8, &w));
+                run("sptmm-delta(check)", w, false);
+            }
+        }
+        bool pass = done.size() >= 2;
+        double worst = 0;
+        for (size_t i = 1; i < done.size(); ++i) {
+            if (act == 0) {
+                pass &= done[i].result == done[0].result;
+            } else {
+                const float *a = (const float *)done[0].result.data(), *b = (const float *)done[i].result.data();
+                for (size_t j = 0; j < (size_t)M * N; ++j) {
+                    double scale = std::max<double>(std::fabs(a[j]), std::sqrt((double)S));
+                    worst = std::max(worst, std::fabs((double)a[j] - b[j]) / scale);
+                }
+                pass &= worst <= 1e-3;
+            }
+        }
+        printf("# check=%s (", pass ? "PASS" : "FAIL");
+        for (size_t i = 0; i < done.size(); ++i) printf("%s%s", i ? (act == 0 ? " == " : " ~ ") : "", done[i].label);
+        if (act != 0) printf("; max rel diff %.2e", worst);
+        printf(")\n");
+        if (!pass) status = 2;
+    }
+    for (auto &m : done) sptmm_weights_free(m.w);
+    sptmm_stream_destroy(stream);
+    sptmm_free(x_d);
+    sptmm_free(c_d);
+    return status;
+}
