@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """Headline benchmark: SpTMM split-K=32 GEMV at M=1, K=6912, N=2560, S=4096 on one MI355X.
 
-A step is one GEMV launch through the C ABI (sptmm_gemv_i8 on the u16-list
-stream).  Launch i reads device copy i % COPIES of the same matrix; the copies
-together exceed the 256 MB last-level cache, so every step streams its 21 MB of
-row indices from HBM ("cold"), as a decoder that walks through gigabytes of
-layer weights does.  The same loop over a single copy ("warm", the reference's
-protocol, main.cu:994-1459) and the other two encodings are reported beside it.
+A step is one launch of the C ABI's sptmm_gemv_i8_batched: 32 independent
+GEMVs of the headline shape, each on its own device copy of the u16-list stream.
+The copies together (671 MB) exceed the 256 MB last-level cache, so every GEMV
+streams its 21 MB of row indices from HBM ("cold"), as a decoder walking
+through gigabytes of layer weights does, and the dispatch latency is paid once
+per step instead of once per GEMV.  Reported beside it: one GEMV per launch
+(cold; warm = the reference's protocol, main.cu:994-1459; and with its per-call
+host sync) and the other two encodings.
 
 Prints ONE JSON line (see the keys at the bottom).
 """
@@ -21,7 +23,7 @@ sys.path.insert(0, ROOT)
 
 METRIC = "µs/GEMV and achieved HBM GB/s (% roofline) at M=1 K=6912 N=2560 S=4096"
 K, N, S, M, SPLIT = 6912, 2560, 4096, 1, 32
-COPIES = 32  # 32 x 21 MB = 671 MB of index streams > 256 MB Infinity Cache
+BATCH = 32  # GEMVs per launch = device copies of the stream: 32 x 21 MB = 671 MB > 256 MB Infinity Cache
 PEAK_GBPS = 8000.0
 
 
@@ -66,9 +68,13 @@ def cpu_baseline(sp_lists, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4096)
-    ap.add_argument("--warmup", type=int, default=256)
+    ap.add_argument("--steps", type=int, default=256, help="timed steps; one step = one launch of BATCH GEMVs")
+    ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--legs", default="single,others",
+                    help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, "
+                         "sync-each-call), others (delta and i2s encodings), copy (4 launches of a 1 GiB copy kernel, for counter "
+                         "calibration); profiling runs use --legs none or --legs copy")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported "
@@ -79,71 +85,104 @@ def main():
     import sptmm_amd as sp
 
     info = sp.device_init(0)
-    _, pos, neg = sp.generate_ternary(K, N, S)
-    Wd, _, _ = sp.generate_ternary(K, N, S, dense=True)
+    Wd, pos, neg = sp.generate_ternary(K, N, S, dense=True)
     X = sp.make_x_i8(0xC0FFEE ^ M, M, K)
     xb = sp.DeviceBuffer.from_numpy(X)
-    cb = sp.DeviceBuffer(4 * M * N)
+    cb = sp.DeviceBuffer(4 * M * N * BATCH)
     st = sp.Stream()
+    legs = set(a.legs.split(","))
 
-    def timed(weights, steps, warmup, mode=0):
-        """-> (us per launch from HIP events on the launch stream, host wall-clock ms per step)."""
+    def timed(weights, launches, warmup, mode):
+        """-> (us per GEMV from two HIP events on the launch stream, host wall-clock ms per launch)."""
+        per = len(weights) if mode == 3 else 1
         if warmup > 0:
-            sp.measure_gemv(weights, 0, xb, M, cb, warmup, mode, st)
+            sp.measure_gemv(weights, 0, xb, M, cb, warmup * per, mode, st)
         sp.device_sync()
         t0 = time.perf_counter()
-        us = sp.measure_gemv(weights, 0, xb, M, cb, steps, mode, st)
+        us = sp.measure_gemv(weights, 0, xb, M, cb, launches * per, mode, st)
         sp.device_sync()
-        return us, (time.perf_counter() - t0) * 1e3 / steps
+        return us, (time.perf_counter() - t0) * 1e3 / launches
 
     w = sp.Weights.upload_u16(pos, neg, K, SPLIT)
-    copies = [w] + [w.clone() for _ in range(COPIES - 1)]
+    copies = [w] + [w.clone() for _ in range(BATCH - 1)]
     nbytes = algorithmic_bytes(w.nbytes)
 
-    # correctness of what is about to be timed (every copy), against the other two encodings
+    # correctness of what is about to be timed: every copy, through the batched entry point
     ref = w.matmul(X)
-    for c in copies[1:]:
-        c.gemv_i8(xb, M, cb, st)
-        st.sync()
-        assert (cb.to_numpy(np.int32, (M, N)) == ref).all()
+    outs = [sp.DeviceBuffer(4 * M * N) for _ in copies]
+    sp.gemv_i8_batched(copies, [xb] * BATCH, outs, M, st)
+    st.sync()
+    for o in outs:
+        assert (o.to_numpy(np.int32, (M, N)) == ref).all()
+        o.free()
 
-    cold_us, cold_ms_step = timed(copies, a.steps, a.warmup)
-    warm_us, _ = timed(copies[:1], a.steps, a.warmup)
-    sync_us, _ = timed(copies[:1], min(a.steps, 2000), 50, mode=1)
+    # headline: EXACTLY --steps launches, each BATCH independent config-0 GEMVs over BATCH distinct
+    # device copies of the stream (671 MB per launch: nothing survives in the 256 MB last-level cache)
+    us_gemv, ms_step = timed(copies, a.steps, a.warmup, 3)
+    launch_us = us_gemv * BATCH
+
+    single = {}
+    if "single" in legs:
+        n1 = 4096
+        single = {
+            "cold_us": round(timed(copies, n1, 256, 0)[0], 3),   # one GEMV per launch, rotating over the copies
+            "warm_us": round(timed(copies[:1], n1, 256, 0)[0], 3),  # same stream every launch (reference protocol)
+            "sync_each_call_us": round(timed(copies[:1], 2000, 50, 1)[0], 3),  # + host sync per launch (main.cu:1456)
+        }
+        single["cold_gbps"] = round(nbytes / single["cold_us"] / 1e3, 1)
+        single["warm_gbps"] = round(nbytes / single["warm_us"] / 1e3, 1)
     for c in copies[1:]:
         c.free()
 
-    others = {}
-    for name, ww in (("delta8_split32", sp.Weights.upload_delta(pos, neg, K, SPLIT)), ("i2s", sp.Weights.upload_i2s(Wd))):
-        assert (ww.matmul(X) == ref).all(), name
-        cps = [ww] + [ww.clone() for _ in range(COPIES * (4 if name == "i2s" else 2) - 1)]
-        c_us, _ = timed(cps, a.steps, a.warmup)
-        w_us, _ = timed(cps[:1], a.steps, a.warmup)
-        b = algorithmic_bytes(ww.nbytes)
-        others[name] = {"cold_us": round(c_us, 3), "warm_us": round(w_us, 3), "bytes": b,
-                        "cold_gbps": round(b / c_us / 1e3, 1), "warm_gbps": round(b / w_us / 1e3, 1)}
-        for c in cps:
-            c.free()
+    if "copy" in legs:
+        # plain copy kernel of known size: the yardstick the traffic counters are scaled by
+        nb = 1 << 30
+        src, dst = sp.DeviceBuffer(nb), sp.DeviceBuffer(nb)
+        src.fill(1)
+        for _ in range(4):
+            sp.copy_kernel(dst, src, nb, st)
+        st.sync()
+        src.free()
+        dst.free()
 
+    others = {}
+    if "others" in legs:
+        for name, mk in (("delta8_split32", lambda: sp.Weights.upload_delta(pos, neg, K, SPLIT)),
+                         ("i2s", lambda: sp.Weights.upload_i2s(Wd))):
+            ww = mk()
+            assert (ww.matmul(X) == ref).all(), name
+            cps = [ww] + [ww.clone() for _ in range(BATCH * (4 if name == "i2s" else 2) - 1)]
+            b = algorithmic_bytes(ww.nbytes)
+            r = {"bytes": b, "single_cold_us": round(timed(cps, 4096, 256, 0)[0], 3),
+                 "single_warm_us": round(timed(cps[:1], 4096, 256, 0)[0], 3)}
+            if name != "i2s":
+                r["batched_cold_us"] = round(timed(cps[:BATCH], a.steps, a.warmup, 3)[0], 3)
+                r["batched_cold_gbps"] = round(b / r["batched_cold_us"] / 1e3, 1)
+            others[name] = r
+            for c in cps:
+                c.free()
+
+    gbps = nbytes / us_gemv / 1e3
     out = {
-        "metric": METRIC, "value": round(cold_us, 3), "unit": "us/GEMV", "n_gpus": 1,
-        "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(cold_ms_step, 6),
+        "metric": METRIC, "value": round(us_gemv, 3), "unit": "us/GEMV", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_step, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "int32", "data": "synthetic",
-        "config": {"workload": "config 0: SpTMM u16 index lists, split-K=32, single GEMV M=1 K=6912 N=2560 "
-                               "S=4096 (2048 +1 / 2048 -1 rows per column, seed 0xCAFEBABE^col), int8 "
-                               "activations uniform [-127,127] seeded, int32 accumulate",
-                   "M": M, "K": K, "N": N, "S": S, "split_k": SPLIT, "weight_copies_rotated": COPIES,
-                   "protocol": "back-to-back launches on one stream between two HIP events, no sync inside"},
-        "hbm_gbps": round(nbytes / cold_us / 1e3, 1), "pct_roofline": round(100 * nbytes / cold_us / 1e3 / PEAK_GBPS, 2),
-        "warm_us": round(warm_us, 3), "warm_gbps": round(nbytes / warm_us / 1e3, 1),
-        "sync_each_call_us": round(sync_us, 3),
-        "other_encodings": others,
+        "config": {"workload": "config 0: SpTMM u16 index lists, split-K=32, GEMV M=1 K=6912 N=2560 S=4096 "
+                               "(2048 +1 / 2048 -1 rows per column, seed 0xCAFEBABE^col), int8 activations "
+                               "uniform [-127,127] seeded, int32 accumulate; one step = one "
+                               "sptmm_gemv_i8_batched launch of %d independent GEMVs of this shape, each on its "
+                               "own device copy of the stream (HBM-cold)" % BATCH,
+                   "M": M, "K": K, "N": N, "S": S, "split_k": SPLIT, "gemvs_per_step": BATCH,
+                   "protocol": "launches back to back on one stream between two HIP events; value = event time "
+                               "/ (steps * gemvs_per_step)"},
+        "hbm_gbps": round(gbps, 1), "pct_roofline": round(100 * gbps / PEAK_GBPS, 2),
+        "single_launch": single, "other_encodings": others,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
-        "roofline": {"bound": "hbm", "achieved": round(nbytes / cold_us / 1e3, 1), "peak": PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(nbytes / cold_us / 1e3 / PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "lists_kernel<int8,1,u16>", "algorithmic_bytes_per_launch": nbytes,
-                     "avg_launch_us": round(cold_us, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "lists_kernel_batched<int8, MT=1, u16>", "launch_us": round(launch_us, 2),
+                     "algorithmic_bytes_per_launch": nbytes * BATCH},
     }
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline((pos, neg))

@@ -137,6 +137,15 @@ int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X_dev, int M, int32_t *C
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X_dev, int M, float *C_dev, void *stream);
 int sptmm_gemv_f32(const sptmm_weights *w, const float *X_dev, int M, float *C_dev, void *stream);
 
+/* `count` independent GEMVs of one shape in ONE launch: C[i] = X[i] . ws[i]
+ * (int8 activations, u16 or gap streams that agree in K, N, S, split_k).  What a
+ * decoder does with projections that share a shape; the reference launches its
+ * kernels one at a time (main.cu:994-1459), so every launch there pays the
+ * dispatch latency that this call pays once.  The pointer arrays are host
+ * arrays of device pointers. */
+int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X_dev, int32_t *const *C_dev, int count,
+                          int M, void *stream);
+
 /* Thin device-memory / stream / event helpers so callers need no HIP headers
  * (the cudaMalloc/cudaMemcpy/cudaEvent* calls of main.cu:767-782, 804-815). */
 int sptmm_malloc(void **dev_ptr, size_t bytes);
@@ -159,7 +168,8 @@ int sptmm_event_elapsed_us(void *start, void *stop, double *us);
  * cache).  act: 0 int8, 1 fp16, 2 fp32.  mode: 0 = back-to-back launches on one
  * stream between two events; 1 = stream synchronize after every launch, as the
  * reference does (main.cu:1456); 2 = one rotation captured into a HIP graph and
- * replayed.  `stream` must come from sptmm_stream_create; the call returns after
+ * replayed; 3 = every rotation is ONE sptmm_gemv_i8_batched launch of all n_ws
+ * GEMVs (C_dev must then hold n_ws * M * N outputs).  `stream` must come from sptmm_stream_create; the call returns after
  * the stream has drained.  Reports mean microseconds per launch, taken from two
  * events recorded on that stream. */
 int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X_dev, int M, void *C_dev,

@@ -10,7 +10,7 @@ __all__ = [
     "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel",
-    "device_sync", "measure_gemv", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
+    "device_sync", "measure_gemv", "gemv_i8_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
 
 KIND_U16, KIND_DELTA, KIND_I2S = 1, 2, 3
@@ -25,7 +25,7 @@ EXPORTS = [
     "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_device_init",
     "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_i2s", "sptmm_weights_clone",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
-    "sptmm_gemv_f32", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
+    "sptmm_gemv_f32", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel",
@@ -75,6 +75,7 @@ def lib() -> C.CDLL:
         L.sptmm_weights_clone.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         for n in ("sptmm_gemv_i8", "sptmm_gemv_f16", "sptmm_gemv_f32"):
             getattr(L, n).argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.sptmm_gemv_i8_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
         L.sptmm_free.argtypes = [C.c_void_p]
         L.sptmm_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
@@ -291,6 +292,16 @@ def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuff
         if own:
             stream.destroy()
     return us.value
+
+
+def gemv_i8_batched(weights, Xs, Cs, M: int, stream: "Stream | None" = None):
+    """One launch for len(weights) GEMVs of one shape: Cs[i] = Xs[i] . weights[i] (device buffers)."""
+    n = len(weights)
+    assert len(Xs) == n and len(Cs) == n
+    wa = (C.c_void_p * n)(*[w.handle for w in weights])
+    xa = (C.c_void_p * n)(*[x.ptr for x in Xs])
+    ca = (C.c_void_p * n)(*[c.ptr for c in Cs])
+    _ck(lib().sptmm_gemv_i8_batched(wa, xa, ca, n, M, stream.handle if stream else None))
 
 
 def device_sync():

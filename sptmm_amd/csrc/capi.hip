@@ -82,7 +82,8 @@ int finish_upload(sptmm_weights *w, const std::vector<uint8_t> &host, sptmm_weig
     return SPTMM_OK;
 }
 
-int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *stream, ActType act)
+int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *stream, ActType act, int batch = 0,
+                const void *const *bw = nullptr, const void *const *bx = nullptr, void *const *bc = nullptr)
 {
     if (!w || !X || !C) return fail(SPTMM_ERR_INVALID, "null pointer");
     if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
@@ -104,6 +105,10 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.index_shift = w->info.kind == SPTMM_KIND_U16 ? u16_index_shift(w->info.K) : 0;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
+    a.batch = batch;
+    a.batch_w = bw;
+    a.batch_X = bx;
+    a.batch_C = bc;
     switch (w->info.kind) {
     case SPTMM_KIND_U16: return launch_u16(a, act, stream);
     case SPTMM_KIND_DELTA: return launch_delta(a, act, stream);
@@ -223,6 +228,26 @@ int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X, int M, int32_t *C, vo
     return gemv_common(w, X, M, C, stream, ACT_I8);
 }
 
+int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X, int32_t *const *C, int count, int M,
+                          void *stream)
+{
+    if (!ws || !X || !C || count < 1) return fail(SPTMM_ERR_INVALID, "bad argument");
+    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    std::vector<const void *> wp(count), xp(count);
+    std::vector<void *> cp(count);
+    for (int i = 0; i < count; ++i) {
+        if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
+        const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
+        if (b.kind == SPTMM_KIND_I2S) return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take u16 or gap streams");
+        if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits)
+            return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);
+        wp[i] = ws[i]->dev;
+        xp[i] = X[i];
+        cp[i] = C[i];
+    }
+    return gemv_common(ws[0], X[0], M, C[0], stream, ACT_I8, count, wp.data(), xp.data(), cp.data());
+}
+
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X, int M, float *C, void *stream)
 {
     return gemv_common(w, X, M, C, stream, ACT_F16);
@@ -317,7 +342,8 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
                        int mode, void *stream, double *us_per_call)
 {
     if (!ws || n_ws < 1 || !X || !C || iters < 1 || !us_per_call) return fail(SPTMM_ERR_INVALID, "bad argument");
-    if (act < ACT_I8 || act > ACT_F32 || mode < 0 || mode > 2) return fail(SPTMM_ERR_INVALID, "bad act or mode");
+    if (act < ACT_I8 || act > ACT_F32 || mode < 0 || mode > 3) return fail(SPTMM_ERR_INVALID, "bad act or mode");
+    if (mode == 3 && act != ACT_I8) return fail(SPTMM_ERR_UNSUPPORTED, "batched timing takes int8 activations");
     if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_measure_gemv needs a stream made by sptmm_stream_create");
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -349,6 +375,21 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
         M_TRY(hipStreamSynchronize(st));
         M_TRY(hipEventRecord(e0, st));
         for (int r = 0; r < reps; ++r) M_TRY(hipGraphLaunch(exec, st));
+        M_TRY(hipEventRecord(e1, st));
+        M_TRY(hipEventSynchronize(e1));
+        M_TRY(hipEventElapsedTime(&ms, e0, e1));
+        *us_per_call = (double)ms * 1000.0 / ((double)reps * n_ws);
+    } else if (mode == 3) {
+        // one launch per rotation: all n_ws GEMVs in a single batched dispatch, outputs side by side in C
+        std::vector<const int8_t *> xs(n_ws, (const int8_t *)X);
+        std::vector<int32_t *> cs(n_ws);
+        for (int i = 0; i < n_ws; ++i) cs[i] = (int32_t *)C + (size_t)i * M * ws[0]->info.N;
+        const int reps = (iters + n_ws - 1) / n_ws;
+        M_TRY(hipEventRecord(e0, st));
+        for (int r = 0; r < reps; ++r) {
+            rc = sptmm_gemv_i8_batched(ws, xs.data(), cs.data(), n_ws, M, st);
+            if (rc != SPTMM_OK) goto done;
+        }
         M_TRY(hipEventRecord(e1, st));
         M_TRY(hipEventSynchronize(e1));
         M_TRY(hipEventElapsedTime(&ms, e0, e1));

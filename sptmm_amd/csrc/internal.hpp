@@ -51,6 +51,11 @@ struct GemvArgs {
     int index_shift;    // u16 stream: fields are row << index_shift
     int compute_units;
     int lds_limit;
+    // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each
+    int batch = 0;
+    const void *const *batch_w = nullptr;
+    const void *const *batch_X = nullptr;
+    void *const *batch_C = nullptr;
 };
 enum ActType { ACT_I8 = 0, ACT_F16 = 1, ACT_F32 = 2 };
 

@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdlib>
 
 #include "internal.hpp"
 
@@ -115,7 +116,7 @@ __device__ __forceinline__ float h2f(u32 d, int hi) { return (float)__builtin_bi
 // can be issued ahead of the weight-stream loads and consumed behind them.
 template <typename Act, int MT> struct Stager {
     static constexpr int NLOAD = MT * (int)sizeof(Act);  // 16-byte loads per item
-    static constexpr int XI = NLOAD >= 8 ? 1 : (NLOAD >= 2 ? 2 : 4);
+    static constexpr int XI = NLOAD >= 8 ? 1 : 2;       // items per thread staged ahead of the stream (more fall to a loop)
 
     static __device__ __forceinline__ void load(const Act *X, int M, int K, int m0, int item, uint4 (&r)[NLOAD])
     {
@@ -477,6 +478,37 @@ __global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel(ListParams 
     B::template run<0>(p, smem);
 }
 
+// Several independent GEMVs of one shape in one launch: blockIdx.z picks the
+// (stream, activations, output) triple, everything else is the kernel above.
+constexpr int BATCH_MAX = 32;
+struct BatchPtrs {
+    const uint8_t *w[BATCH_MAX];
+    const void *X[BATCH_MAX];
+    void *C[BATCH_MAX];
+};
+
+template <typename Act, int MT, int MODE, bool PRE, bool FIXED>
+__global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel_batched(ListParams p, BatchPtrs b)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    typedef ListsBody<Act, MT, MODE, PRE> B;
+    p.w = b.w[blockIdx.z];
+    p.X = b.X[blockIdx.z];
+    p.C = b.C[blockIdx.z];
+    if constexpr (FIXED) {
+        switch (p.n_lane / B::E16) {
+        case 1: B::template run<1>(p, smem); return;
+        case 2: B::template run<2>(p, smem); return;
+        case 3: B::template run<3>(p, smem); return;
+        case 4: B::template run<4>(p, smem); return;
+        case 6: B::template run<6>(p, smem); return;
+        case 8: B::template run<8>(p, smem); return;
+        default: break;
+        }
+    }
+    B::template run<0>(p, smem);
+}
+
 // ------------------------------------------------------------------- i2s GEMV
 struct I2sParams {
     const uint4 *w;
@@ -608,10 +640,13 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
     // CU gets more than LISTS_MAX_WAVES tasks pick the count that wastes the
     // fewest wavefront slots over the task loop.
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
+    static const int tune_wpb = getenv("SPTMM_WAVES_PER_WG") ? atoi(getenv("SPTMM_WAVES_PER_WG")) : 0;
+    static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 1;
+    const int slots = cus * (tune_wgs > 0 ? tune_wgs : 1);  // workgroups resident at once
     int wpb = a.W, best = 1 << 30;
     for (int w = a.W; w <= LISTS_MAX_WAVES; w += a.W) {
         int blocks = (a.tasks + w - 1) / w;
-        int grid = blocks < cus ? blocks : cus;
+        int grid = blocks < slots ? blocks : slots;
         int iters = (blocks + grid - 1) / grid;
         int cost = iters * w;
         if (cost < best || (cost == best && w > wpb)) {
@@ -619,8 +654,9 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
             wpb = w;
         }
     }
+    if (tune_wpb > 0 && tune_wpb <= LISTS_MAX_WAVES && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int blocks = (a.tasks + wpb - 1) / wpb;
-    const int grid_x = blocks < cus ? blocks : cus;
+    const int grid_x = blocks < slots ? blocks : slots;
     const int iters = (blocks + grid_x - 1) / grid_x;
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, a.n_lane, a.tasks, ilog2(a.L), a.W, iters};
     constexpr int SLOT = slot_bytes<Act, MT>();
@@ -628,10 +664,33 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     // straight-line bodies for the int8 paths of the u16 and 8-bit gap streams
     constexpr bool FIXED = sizeof(Act) == 1 && MODE != 2;
+    dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
+    if (a.batch) {
+        if constexpr (sizeof(Act) == 1) {
+            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, FIXED>;
+            static std::atomic<size_t> lds_granted_b{48 * 1024};
+            if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_b)) return rc;
+            for (int first = 0; first < a.batch; first += BATCH_MAX) {
+                BatchPtrs b{};
+                const int n = a.batch - first < BATCH_MAX ? a.batch - first : BATCH_MAX;
+                for (int i = 0; i < n; ++i) {
+                    b.w[i] = (const uint8_t *)a.batch_w[first + i];
+                    b.X[i] = a.batch_X[first + i];
+                    b.C[i] = a.batch_C[first + i];
+                }
+                grid.z = n;
+                hipLaunchKernelGGL(kern, grid, block, lds, st, p, b);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) return hip_fail(e, "lists_kernel_batched launch");
+            }
+            return SPTMM_OK;
+        } else {
+            return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take int8 activations");
+        }
+    }
     auto kern = lists_kernel<Act, MT, MODE, PRE, FIXED>;
     static std::atomic<size_t> lds_granted{48 * 1024};
     if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
-    dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     hipLaunchKernelGGL(kern, grid, block, lds, st, p);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel launch");

@@ -334,3 +334,42 @@ def test_streams_and_clone():
     for o in (w, w2, xb, cb):
         o.free()
     st.destroy()
+
+
+# ------------------------------------------------------------------ batched launch
+@pytest.mark.parametrize("kind", ["u16", "delta"])
+@pytest.mark.parametrize("M,count", [(1, 3), (4, 5), (1, 40)])
+def test_batched_launch_equals_single_launches(kind, M, count):
+    K, N, S = 2560, 640, 1536
+    _, pos, neg = matrix(K, N, S)
+    up = sp.Weights.upload_u16 if kind == "u16" else sp.Weights.upload_delta
+    base = up(pos, neg, K, 32)
+    ws = [base] + [base.clone() for _ in range(count - 1)]
+    Xs = [x_i8(9000 + i, M, K) for i in range(count)]
+    xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
+    cb = [sp.DeviceBuffer(4 * M * N) for _ in range(count)]
+    for c in cb:
+        c.fill(0xFF)
+    say("batched", kind, "M", M, "count", count)
+    st = sp.Stream()
+    sp.gemv_i8_batched(ws, xb, cb, M, st)
+    st.sync()
+    for i in range(count):
+        want = oracle.sptmm_i8_mt(Xs[i], pos, neg, 4)
+        assert (cb[i].to_numpy(np.int32, (M, N)) == want).all(), i
+    for o in ws + xb + cb:
+        o.free()
+    st.destroy()
+
+
+def test_batched_launch_rejects_mixed_shapes():
+    _, pos, neg = matrix(512, 48, 256)
+    a = sp.Weights.upload_u16(pos, neg, 512, 32)
+    b = sp.Weights.upload_u16(pos, neg, 512, 16)
+    xb = sp.DeviceBuffer(512)
+    cb = sp.DeviceBuffer(4 * 48)
+    with pytest.raises(sp.SptmmError) as e:
+        sp.gemv_i8_batched([a, b], [xb, xb], [cb, cb], 1)
+    assert e.value.code == -1
+    for o in (a, b, xb, cb):
+        o.free()
