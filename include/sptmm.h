@@ -56,6 +56,7 @@ typedef struct sptmm_winfo {
     int K, N, S;     /* S = nonzeros per column (0 for i2s) */
     int split_k;     /* lanes cooperating on one column (0 for i2s) */
     int delta_bits;  /* 8 or 16 for SPTMM_KIND_DELTA, else 0 */
+    int delta_layout; /* SPTMM_KIND_DELTA: 1 = contiguous runs, 2 = striped by row mod 32; else 0 */
     uint64_t stream_bytes; /* bytes of the weight stream one GEMV reads */
 } sptmm_winfo;
 
@@ -98,6 +99,22 @@ size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits);
 int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out);
 int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg);
 
+/* Striped gap stream, split_k 32 or 64: lane v of a column owns the rows of one
+ * residue class mod 32 (row = v%32 + 32*j) and stores the gaps of j as bytes, so
+ * the 32 lanes of a half-wavefront always read 32 different LDS banks; the
+ * lists of a wavefront are padded to a common length with entries that land on
+ * zero rows behind the activation tile.  Costs ~30 % more bytes (and 1.5x the
+ * gathers) than the run layout above and removes its bank conflicts; measured
+ * slower than runs on MI355X, so uploads use it only on request.  _eligible returns 1 when every
+ * gap (in units of 32 rows) fits a byte, 0 when not, < 0 on bad arguments.
+ * _bytes returns the size of the stream (0 if not eligible); *read_bytes is
+ * what one GEMV reads of it (tasks are stored at a fixed stride). */
+int sptmm_delta_striped_eligible(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k);
+size_t sptmm_pack_delta_striped_bytes(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k,
+                                      size_t *read_bytes, int *n_min, int *n_max);
+int sptmm_pack_delta_striped(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out);
+int sptmm_unpack_delta_striped(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg);
+
 /* i2s: 16 weights per word, code = w + 2, element e at bit 8*(e%4) + 2*(e/4)
  * (main.cu:176-192, decode bitnet_kernels.cuh:52-72).  Word order is this
  * library's own wave64 tiling, not the reference's (whose prepared matrix,
@@ -117,6 +134,9 @@ int sptmm_device_init(int device, sptmm_devinfo *out);
  * prepareW_map / prepareW_i2s sequence of main.cu:914-989 and 1851-1859. */
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
+/* layout: 0 = default (runs), 1 = runs, 2 = striped (kept as an alternative; slower where measured) */
+int sptmm_weights_upload_delta_layout(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int layout,
+                                      sptmm_weights **out);
 int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weights **out);
 /* Second device copy of the same stream (used to rotate over more bytes than
  * the last-level cache holds when timing cold reads). */

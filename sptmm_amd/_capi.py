@@ -8,7 +8,8 @@ import numpy as np
 
 __all__ = [
     "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
-    "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s",
+    "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "delta_striped_eligible",
+    "pack_delta_striped", "unpack_delta_striped", "pack_i2s", "unpack_i2s",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel",
     "device_sync", "measure_gemv", "gemv_i8_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
@@ -21,9 +22,11 @@ _LIB = None
 EXPORTS = [
     "sptmm_last_error", "sptmm_version", "sptmm_generate_ternary", "sptmm_lists_from_dense", "sptmm_make_x_i8",
     "sptmm_pack_u16_bytes", "sptmm_pack_u16", "sptmm_unpack_u16", "sptmm_delta_bits", "sptmm_pack_delta_bytes",
-    "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
+    "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_delta_striped_eligible", "sptmm_pack_delta_striped_bytes",
+    "sptmm_pack_delta_striped", "sptmm_unpack_delta_striped", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
     "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_device_init",
-    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_i2s", "sptmm_weights_clone",
+    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_delta_layout",
+    "sptmm_weights_upload_i2s", "sptmm_weights_clone",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
     "sptmm_gemv_f32", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
@@ -46,7 +49,7 @@ class DevInfo(C.Structure):
 
 class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
-                ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64)]
+                ("delta_bits", C.c_int), ("delta_layout", C.c_int), ("stream_bytes", C.c_uint64)]
 
 
 def lib_path() -> str:
@@ -64,7 +67,8 @@ def lib() -> C.CDLL:
         L = C.CDLL(p)
         L.sptmm_last_error.restype = C.c_char_p
         L.sptmm_version.restype = C.c_char_p
-        for n in ("sptmm_pack_u16_bytes", "sptmm_pack_delta_bytes", "sptmm_pack_i2s_bytes", "sptmm_weights_bytes"):
+        for n in ("sptmm_pack_u16_bytes", "sptmm_pack_delta_bytes", "sptmm_pack_i2s_bytes", "sptmm_weights_bytes",
+                  "sptmm_pack_delta_striped_bytes"):
             getattr(L, n).restype = C.c_size_t
         L.sptmm_i2s_pack_word.restype = C.c_uint32
         L.sptmm_i2s_decode_word.restype = None
@@ -174,6 +178,30 @@ def unpack_delta(packed, K, N, S, split_k, bits):
     pos = np.empty((N, S // 2), np.uint16)
     neg = np.empty((N, S // 2), np.uint16)
     _ck(lib().sptmm_unpack_delta(_p(packed), K, N, S, split_k, bits, _p(pos), _p(neg)))
+    return pos, neg
+
+
+def delta_striped_eligible(pos, neg, K, split_k) -> bool:
+    N, half = pos.shape
+    return bool(_ck(lib().sptmm_delta_striped_eligible(_p(pos), _p(neg), K, N, 2 * half, split_k)))
+
+
+def pack_delta_striped(pos, neg, K, split_k):
+    """-> (stream bytes, dict(read_bytes, n_min, n_max))."""
+    N, half = pos.shape
+    rb, lo, hi = C.c_size_t(), C.c_int(), C.c_int()
+    n = lib().sptmm_pack_delta_striped_bytes(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(rb), C.byref(lo), C.byref(hi))
+    if not n:
+        raise SptmmError(-2, "matrix not eligible for the striped gap layout")
+    out = np.zeros(n, np.uint8)
+    _ck(lib().sptmm_pack_delta_striped(_p(pos), _p(neg), K, N, 2 * half, split_k, _p(out)))
+    return out, {"read_bytes": rb.value, "n_min": lo.value, "n_max": hi.value}
+
+
+def unpack_delta_striped(packed, K, N, S, split_k):
+    pos = np.empty((N, S // 2), np.uint16)
+    neg = np.empty((N, S // 2), np.uint16)
+    _ck(lib().sptmm_unpack_delta_striped(_p(packed), K, N, S, split_k, _p(pos), _p(neg)))
     return pos, neg
 
 
@@ -326,10 +354,11 @@ class Weights:
         return cls(h)
 
     @classmethod
-    def upload_delta(cls, pos, neg, K, split_k) -> "Weights":
+    def upload_delta(cls, pos, neg, K, split_k, layout: int = 0) -> "Weights":
+        """layout: 0 / 1 = contiguous runs (default), 2 = striped by row mod 32 (alternative, slower where measured)."""
         N, half = pos.shape
         h = C.c_void_p()
-        _ck(lib().sptmm_weights_upload_delta(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(h)))
+        _ck(lib().sptmm_weights_upload_delta_layout(_p(pos), _p(neg), K, N, 2 * half, split_k, layout, C.byref(h)))
         return cls(h)
 
     @classmethod

@@ -27,10 +27,26 @@ def _run(cmd):
         print(out, file=sys.stderr)
 
 
+SOURCES = ("formats.cpp", "capi.hip", "i2s.hip", "lists_u16_scaled.hip", "lists_u16_plain.hip", "lists_runs8.hip",
+           "lists_runs16.hip", "lists_striped.hip")
+
+
 def build_lib() -> str:
-    srcs = [os.path.join(CSRC, f) for f in ("formats.cpp", "kernels.hip", "capi.hip")]
+    """One translation unit per stream flavour, compiled side by side, then linked."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(f):
+        obj = os.path.join(objdir, f + ".o")
+        _run([HIPCC, *HIPFLAGS, "-c", "-o", obj, "-x", "hip", os.path.join(CSRC, f)])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
     tmp = LIB + ".tmp"
-    _run([HIPCC, *HIPFLAGS, "-shared", "-pthread", "-o", tmp, "-x", "hip", *srcs])
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-pthread", "-o", tmp, *objs])
     os.replace(tmp, LIB)
     return LIB
 

@@ -1,0 +1,203 @@
+// i2s (2-bit packed dense ternary) GEMV, the copy kernel, and the dispatch of the
+// list-stream launchers that live in their own translation units.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "internal.hpp"
+
+namespace sptmm {
+
+typedef unsigned int u32;
+
+template <int CTRL> __device__ __forceinline__ int dpp(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
+__device__ __forceinline__ int swz16(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401f); }  // lane ^ 16
+
+// Sum over groups of 2^logL consecutive lanes (logL >= 2); every lane of a group ends with the group's total.
+__device__ __forceinline__ int lanes_sum(int v, int logL)
+{
+    v += dpp<0xB1>(v);                   // quad_perm [1,0,3,2]
+    v += dpp<0x4E>(v);                   // quad_perm [2,3,0,1]
+    if (logL >= 3) v += dpp<0x141>(v);   // row_half_mirror
+    if (logL >= 4) v += dpp<0x140>(v);   // row_mirror
+    if (logL >= 5) v += swz16(v);
+    if (logL >= 6) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// ------------------------------------------------------------------- i2s GEMV
+struct I2sParams {
+    const uint4 *w;
+    const int8_t *X;
+    int *C;
+    int M, K, Kp, N, rounds;
+};
+
+// Workgroup = 16 columns; wavefront `wave` takes rounds wave, wave+waves, ...;
+// in a round lane (col%16)*4 + q reads 64 weights (rows 256*r + 64*q ...) of its column.
+// Codes 1..3 are used as they are in dot4; the "-2" of the decode
+// (bitnet_kernels.cuh:70) becomes one subtraction of 2*sum(X row) at the end.
+template <int MT>
+__global__ void __launch_bounds__(1024) i2s_kernel(I2sParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    int8_t *lx = reinterpret_cast<int8_t *>(smem);                       // [MT][Kp]
+    int *part = reinterpret_cast<int *>(smem + (size_t)MT * p.Kp);      // [waves][16][MT]
+    int *sums = part + (blockDim.x >> 6) * 16 * MT;                      // [waves][MT]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int grp = blockIdx.x, m0 = blockIdx.y * MT;
+    constexpr int RPB = 4;
+
+    uint4 wv[RPB];
+#pragma unroll
+    for (int i = 0; i < RPB; ++i) {
+        int r = wave + i * waves;
+        wv[i] = (r < p.rounds) ? p.w[((size_t)grp * p.rounds + r) * 64 + lane] : make_uint4(0, 0, 0, 0);
+    }
+
+    // stage X rows (zero beyond M and beyond K) and accumulate the row sums on the way
+    int rs[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        rs[m] = 0;
+        const uint4 *src = reinterpret_cast<const uint4 *>(p.X + (size_t)(m0 + m) * p.K);
+        uint4 *dst = reinterpret_cast<uint4 *>(lx + (size_t)m * p.Kp);
+        for (int i = tid; i < p.Kp / 16; i += blockDim.x) {
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (m0 + m < p.M && i < p.K / 16) v = src[i];
+            dst[i] = v;
+            rs[m] = __builtin_amdgcn_sdot4((int)v.x, 0x01010101, rs[m], false);
+            rs[m] = __builtin_amdgcn_sdot4((int)v.y, 0x01010101, rs[m], false);
+            rs[m] = __builtin_amdgcn_sdot4((int)v.z, 0x01010101, rs[m], false);
+            rs[m] = __builtin_amdgcn_sdot4((int)v.w, 0x01010101, rs[m], false);
+        }
+        rs[m] = lanes_sum(rs[m], 6);
+        if (lane == 0) sums[wave * MT + m] = rs[m];
+    }
+    __syncthreads();
+
+    int acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = 0;
+    const int q = lane & 3;
+
+    for (int r0 = wave;; r0 += RPB * waves) {
+#pragma unroll
+        for (int i = 0; i < RPB; ++i) {
+            const int r = r0 + i * waves;
+            if (r < p.rounds) {
+                const u32 words[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+                    const uint4 *xr = reinterpret_cast<const uint4 *>(lx + (size_t)m * p.Kp + 256 * r + 64 * q);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint4 x = xr[j];
+                        const u32 wd = words[j];
+                        acc[m] = __builtin_amdgcn_sdot4((int)x.x, (int)(wd & 0x03030303u), acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4((int)x.y, (int)((wd >> 2) & 0x03030303u), acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4((int)x.z, (int)((wd >> 4) & 0x03030303u), acc[m], false);
+                        acc[m] = __builtin_amdgcn_sdot4((int)x.w, (int)((wd >> 6) & 0x03030303u), acc[m], false);
+                    }
+                }
+            }
+        }
+        if (r0 + RPB * waves >= p.rounds) break;
+#pragma unroll
+        for (int i = 0; i < RPB; ++i) {
+            int r = r0 + (RPB + i) * waves;
+            wv[i] = (r < p.rounds) ? p.w[((size_t)grp * p.rounds + r) * 64 + lane] : make_uint4(0, 0, 0, 0);
+        }
+    }
+
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        acc[m] = lanes_sum(acc[m], 2);
+        if (q == 0) part[(wave * 16 + (lane >> 2)) * MT + m] = acc[m];
+    }
+    __syncthreads();
+    for (int t = tid; t < 16 * MT; t += blockDim.x) {
+        const int col = t / MT, m = t % MT;
+        int s = 0, sx = 0;
+        for (int w = 0; w < waves; ++w) {
+            s += part[(w * 16 + col) * MT + m];
+            sx += sums[w * MT + m];
+        }
+        if (m0 + m < p.M) p.C[(size_t)(m0 + m) * p.N + grp * 16 + col] = s - 2 * sx;
+    }
+}
+
+__global__ void __launch_bounds__(256) copy_kernel(uint4 *dst, const uint4 *src, size_t n16)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+// ------------------------------------------------------------------ launchers
+static int hip_fail(hipError_t e, const char *what)
+{
+    return fail(SPTMM_ERR_HIP, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+}
+
+// Dynamic LDS above the default cap has to be granted per kernel once.
+static int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &granted)
+{
+    if (lds <= granted.load(std::memory_order_relaxed)) return SPTMM_OK;
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    granted.store(lds, std::memory_order_relaxed);
+    return SPTMM_OK;
+}
+
+template <int MT>
+static int launch_i2s_t(const GemvArgs &a, hipStream_t st, int waves)
+{
+    const int Kp = i2s_padded_k(a.K);
+    I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256};
+    size_t lds = (size_t)MT * Kp + (size_t)waves * 16 * MT * 4 + (size_t)waves * MT * 4;
+    auto kern = i2s_kernel<MT>;
+    static std::atomic<size_t> lds_granted{48 * 1024};
+    if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
+    dim3 grid(a.N / 16, (a.M + MT - 1) / MT), block(64 * waves);
+    hipLaunchKernelGGL(kern, grid, block, lds, st, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? SPTMM_OK : hip_fail(e, "i2s_kernel launch");
+}
+
+int launch_i2s(const GemvArgs &a, void *stream)
+{
+    const int Kp = i2s_padded_k(a.K), rounds = Kp / 256, groups = a.N / 16;
+    int rpw = groups >= 2 * a.compute_units ? 4 : (groups >= a.compute_units ? 2 : 1);
+    int waves = (rounds + rpw - 1) / rpw;
+    waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
+    const size_t extra = (size_t)waves * 17 * 4;
+    hipStream_t st = (hipStream_t)stream;
+    if (a.M >= 5 && (size_t)8 * Kp + extra * 8 <= (size_t)a.lds_limit) return launch_i2s_t<8>(a, st, waves);
+    if (a.M >= 2 && (size_t)4 * Kp + extra * 4 <= (size_t)a.lds_limit) return launch_i2s_t<4>(a, st, waves);
+    if ((size_t)Kp + extra > (size_t)a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "K too large for the LDS activation tile");
+    return launch_i2s_t<1>(a, st, waves);
+}
+
+int launch_copy(void *dst, const void *src, size_t bytes, void *stream)
+{
+    if (bytes % 16) return fail(SPTMM_ERR_INVALID, "copy size must be a multiple of 16 bytes");
+    size_t n16 = bytes / 16;
+    int blocks = (int)((n16 + 255) / 256 < 256 * 64 ? (n16 + 255) / 256 : 256 * 64);
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint4 *)dst, (const uint4 *)src, n16);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? SPTMM_OK : hip_fail(e, "copy_kernel launch");
+}
+
+int launch_u16(const GemvArgs &a, ActType act, void *stream)
+{
+    return a.index_shift == 2 ? launch_u16_scaled(a, act, stream) : launch_u16_plain(a, act, stream);
+}
+
+int launch_delta(const GemvArgs &a, ActType act, void *stream)
+{
+    if (a.delta_layout == 2) return launch_striped(a, act, stream);
+    return a.delta_bits == 8 ? launch_runs8(a, act, stream) : launch_runs16(a, act, stream);
+}
+
+}  // namespace sptmm

@@ -35,6 +35,10 @@ size_t slot_offset(int n_lane, int esz, int sign, int lane, int j);
 // u16 stream fields are row indices shifted left by this many bits (2 when 4*K fits 16 bits).
 int u16_index_shift(int K);
 
+// striped gap stream (formats.cpp): stride between tasks, smallest / largest per-task entry count
+struct StripedPlan;
+int striped_plan(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, StripedPlan *pl);
+
 // i2s tiling: 16 columns x 4 lanes per wave-load, 16 bytes (64 weights) per lane.
 inline int i2s_padded_k(int K) { return (K + 255) / 256 * 256; }
 
@@ -48,6 +52,10 @@ struct GemvArgs {
     void *C;            // device output, row-major [M][N]
     int M, K, N, half, split_k, n_lane, tasks, L, G, W;
     int delta_bits;
+    int delta_layout;   // 1 = contiguous runs, 2 = striped by row mod 32
+    int task_stride;    // striped: bytes between tasks
+    int n_min;          // striped: smallest per-task entry count
+    int n_max;          // striped: largest per-task entry count
     int index_shift;    // u16 stream: fields are row << index_shift
     int compute_units;
     int lds_limit;
@@ -60,6 +68,11 @@ struct GemvArgs {
 enum ActType { ACT_I8 = 0, ACT_F16 = 1, ACT_F32 = 2 };
 
 int launch_u16(const GemvArgs &a, ActType act, void *stream);
+int launch_u16_scaled(const GemvArgs &a, ActType act, void *stream);   // lists_u16_scaled.hip
+int launch_u16_plain(const GemvArgs &a, ActType act, void *stream);    // lists_u16_plain.hip
+int launch_runs8(const GemvArgs &a, ActType act, void *stream);        // lists_runs8.hip
+int launch_runs16(const GemvArgs &a, ActType act, void *stream);       // lists_runs16.hip
+int launch_striped(const GemvArgs &a, ActType act, void *stream);      // lists_striped.hip
 int launch_delta(const GemvArgs &a, ActType act, void *stream);
 int launch_i2s(const GemvArgs &a, void *stream);
 int launch_copy(void *dst, const void *src, size_t bytes, void *stream);

@@ -1,12 +1,8 @@
-// gfx950 kernels of the SpTMM engine and their launchers.
-//
-// All three kernels are HBM-bound gather/unpack work: no multiplies on the
-// list paths, packed-integer dot4 on the i2s path, no MFMA anywhere.  Common
-// shape: the activation tile is staged once per workgroup in LDS (every column
-// reuses it), each 64-lane wavefront streams its slice of the weight stream
-// with 16-byte per-lane loads that are contiguous across the wavefront, and
-// split-K partials are folded across lanes with DPP, then (when a column spans
-// several wavefronts) through a small LDS buffer.  No atomics.
+// Device code and launch templates shared by the list-stream translation units
+// (u16 lists, run gap streams, striped gap streams).  Each .hip file that
+// includes this header instantiates the kernels of one stream flavour, so the
+// flavours compile in parallel.
+#pragma once
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -15,6 +11,7 @@
 #include "internal.hpp"
 
 namespace sptmm {
+
 
 typedef unsigned int u32;
 
@@ -60,25 +57,26 @@ __device__ __forceinline__ void gather(const unsigned char *lds, u32 addr, typen
 }
 
 // MODE 0: fields are u16 row indices (already multiplied by 4 when PRE).
-// MODE 1 / 2: fields are 8- / 16-bit gaps added to a running row index.
-// Consumes the low NBYTES of `d`.
+// MODE 1 / 2: fields are 8- / 16-bit gaps in rows; MODE 3: 8-bit gaps in units
+// of 32 rows (striped stream).  `run` is the byte offset of the current row's
+// slot in the tile.  Consumes the low NBYTES of `d`.
 template <typename Act, int MT, int MODE, bool PRE, bool NEG, int NBYTES>
 __device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &run, typename Acc<Act>::type (&acc)[MT])
 {
     constexpr int SH = ilog2(slot_bytes<Act, MT>());
-    if constexpr (MODE == 1) {
+    if constexpr (MODE == 1 || MODE == 3) {
 #pragma unroll
         for (int b = 0; b < NBYTES; ++b) {
-            run += (d >> (8 * b)) & 0xffu;
-            gather<Act, MT, NEG>(lds, run << SH, acc);
+            run += ((d >> (8 * b)) & 0xffu) << (MODE == 3 ? SH + 5 : SH);
+            gather<Act, MT, NEG>(lds, run, acc);
         }
     } else {
 #pragma unroll
         for (int h = 0; h < NBYTES / 2; ++h) {
             u32 f = h ? (d >> 16) : (d & 0xffffu);
             if constexpr (MODE == 2) {
-                run += f;
-                gather<Act, MT, NEG>(lds, run << SH, acc);
+                run += f << SH;
+                gather<Act, MT, NEG>(lds, run, acc);
             } else {
                 gather<Act, MT, NEG>(lds, f << (PRE ? SH - 2 : SH), acc);
             }
@@ -203,7 +201,8 @@ struct ListParams {
     const void *X;
     void *C;
     int M, K, N;
-    int n_lane, tasks, logL, W;
+    int n_lane, tasks, logL, W;  // n_lane: entries per lane per sign (striped stream: the smallest over all tasks)
+    int task_stride;             // striped stream: bytes between tasks
     int iters;  // tasks each wavefront walks: ceil(tasks / (gridDim.x * waves))
 };
 
@@ -237,11 +236,14 @@ template <typename Act, int MT, int MODE, bool PRE>
 struct ListsBody {
     typedef typename Acc<Act>::type A;
     typedef Stager<Act, MT> St;
-    static constexpr int ESZ = (MODE == 1) ? 1 : 2;   // bytes per stream entry
+    static constexpr int SLOT_OF = slot_bytes<Act, MT>();
+    static constexpr int ESZ = (MODE == 1 || MODE == 3) ? 1 : 2;   // bytes per stream entry
     static constexpr int E16 = 16 / ESZ;              // entries per 16-byte load
-    static constexpr int HDR = MODE ? 256 : 0;        // restart indices of a gap-stream task
-    static constexpr int SLOT = slot_bytes<Act, MT>();
-    static constexpr int CH = 4;                      // rounds per chunk of the generic path
+    static constexpr int HDR = MODE == 3 ? 272 : (MODE ? 256 : 0);  // first rows (and entry count) of a gap-stream task
+    static constexpr int ZROWS = 64;                  // zero slots behind the tile (row K, and the striped stream's padding rows)
+    static constexpr int SH = ilog2(SLOT_OF);
+    static constexpr int SLOT = SLOT_OF;
+    static constexpr int RING = 8;                    // rounds in flight on the generic path
 #ifndef SPTMM_EARLY
 #define SPTMM_EARLY 2
 #endif
@@ -251,22 +253,29 @@ struct ListsBody {
     {
         consume16<Act, MT, MODE, PRE, false>(smem, x.p, runp, acc);
         consume16<Act, MT, MODE, PRE, true>(smem, x.q, runq, acc);
+        // Pin the sums (and the running rows) once per round.  Integer adds may be
+        // reassociated freely, and without this the compiler keeps every gathered
+        // value of every round alive to sum them in one tree at the end.
+#pragma unroll
+        for (int m = 0; m < MT; ++m) asm volatile("" : "+v"(acc[m]));
+        if constexpr (MODE != 0) asm volatile("" : "+v"(runp), "+v"(runq));
     }
 
     // RF > 0: the task has exactly RF full rounds and all of them live in
     // registers, loaded and consumed in straight-line code (so every wait on the
-    // stream is for one round only).  RF == 0: any number of rounds, walked in
-    // double-buffered chunks of CH.
+    // stream is for one round only).  RF == 0: any number of rounds, through a
+    // ring of RING rounds in flight.
     template <int RF>
     static __device__ __forceinline__ void run(const ListParams &p, unsigned char *smem)
     {
-        constexpr int NB = RF > 0 ? RF : 2 * CH;
-        A *part = reinterpret_cast<A *>(smem + (((size_t)(p.K + 1) * SLOT + 15) & ~(size_t)15));
+        constexpr int NB = RF > 0 ? RF : RING;
+        A *part = reinterpret_cast<A *>(smem + (size_t)(p.K + ZROWS) * SLOT);
         const int tid = threadIdx.x, nt = blockDim.x;
         const int lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
         const int m0 = blockIdx.y * MT;
-        const size_t task_bytes = HDR + (size_t)128 * ESZ * p.n_lane;
-        const int R = p.n_lane / E16, nchunk = R / CH;
+        const size_t task_bytes = MODE == 3 ? (size_t)p.task_stride : HDR + (size_t)128 * ESZ * p.n_lane;
+        // striped stream: tasks differ in length; p.n_lane is the shortest, which is all the prologue may assume
+        const int R0 = p.n_lane / E16;
         int task = blockIdx.x * waves + wave;
         const int task_step = gridDim.x * waves;
         const Act *X = reinterpret_cast<const Act *>(p.X);
@@ -291,15 +300,9 @@ struct ListsBody {
             if constexpr (RF > 0) {
 #pragma unroll
                 for (int i = 0; i < (RF < EARLY ? RF : EARLY); ++i) buf[i] = load_round(wp, i);
-            } else {
-                if (nchunk > 0) {
+            } else if (R0 > 0) {
 #pragma unroll
-                    for (int i = 0; i < CH; ++i) buf[i] = load_round(wp, i);
-                }
-                if (nchunk > 1) {
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) buf[CH + i] = load_round(wp, CH + i);
-                }
+                for (int i = 0; i < EARLY; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
             }
         }
 
@@ -311,13 +314,19 @@ struct ListsBody {
             const uint4 *wp = reinterpret_cast<const uint4 *>(p.w + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
 #pragma unroll
             for (int i = EARLY; i < RF; ++i) buf[i] = load_round(wp, i);
+        } else if constexpr (RF == 0) {
+            if (R0 > 0) {
+                const uint4 *wp = reinterpret_cast<const uint4 *>(p.w + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
+#pragma unroll
+                for (int i = EARLY; i < RING; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
+            }
         }
         for (int item = tid + St::XI * nt; item < items; item += nt) {
             uint4 r[St::NLOAD];
             St::load(X, p.M, p.K, m0, item, r);
             St::store(smem, item, r);
         }
-        if (tid < SLOT / 4) reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[tid] = 0u;  // slot K reads as zero
+        for (int i = tid; i < ZROWS * SLOT / 4; i += nt) reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = 0u;  // rows K.. read as zero
         __syncthreads();
 
         A *C = reinterpret_cast<A *>(p.C);
@@ -327,11 +336,14 @@ struct ListsBody {
             const uint8_t *tb = p.w + (size_t)(active ? task : 0) * task_bytes;
             const uint4 *wp = reinterpret_cast<const uint4 *>(tb + HDR) + lane;
             u32 runp = 0, runq = 0;
+            int n_lane = p.n_lane;
             if constexpr (MODE != 0) {
                 const unsigned short *rs = reinterpret_cast<const unsigned short *>(tb);
-                runp = rs[lane];
-                runq = rs[64 + lane];
+                runp = (u32)rs[lane] << SH;
+                runq = (u32)rs[64 + lane] << SH;
             }
+            if constexpr (MODE == 3 && RF == 0) n_lane = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int *>(tb + 256));
+            const int R = n_lane / E16, rem = n_lane - R * E16;
             A acc[MT];
 #pragma unroll
             for (int m = 0; m < MT; ++m) acc[m] = (A)0;
@@ -341,81 +353,91 @@ struct ListsBody {
 #pragma unroll
                     for (int i = 0; i < RF; ++i) buf[i] = load_round(wp, i);
                 }
-#pragma unroll
-                for (int i = 0; i < RF; ++i) eat(smem, buf[i], runp, runq, acc);
             } else {
+                // ring of RING rounds, loads clamped to the task's last round so that they stay unconditional
                 if (it > 0) {
-                    if (nchunk > 0) {
+                    if (R > 0) {
 #pragma unroll
-                        for (int i = 0; i < CH; ++i) buf[i] = load_round(wp, i);
+                        for (int i = 0; i < RING; ++i) buf[i] = load_round(wp, i < R ? i : R - 1);
                     }
-                    if (nchunk > 1) {
+                } else if (MODE == 3) {  // this task may be longer than the shortest one the prologue assumed
 #pragma unroll
-                        for (int i = 0; i < CH; ++i) buf[CH + i] = load_round(wp, CH + i);
-                    }
-                }
-                int c = 0;
-                for (; c + 3 < nchunk; c += 2) {  // steady state: eat a chunk, refill it two chunks ahead
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) eat(smem, buf[i], runp, runq, acc);
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) buf[i] = load_round(wp, (c + 2) * CH + i);
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) eat(smem, buf[CH + i], runp, runq, acc);
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) buf[CH + i] = load_round(wp, (c + 3) * CH + i);
-                }
-                const int left = nchunk - c;  // 0..3 chunks, the first two already in registers
-                if (left >= 1) {
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) eat(smem, buf[i], runp, runq, acc);
-                }
-                if (left == 3) {
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) buf[i] = load_round(wp, (c + 2) * CH + i);
-                }
-                if (left >= 2) {
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) eat(smem, buf[CH + i], runp, runq, acc);
-                }
-                if (left == 3) {
-#pragma unroll
-                    for (int i = 0; i < CH; ++i) eat(smem, buf[i], runp, runq, acc);
-                }
-                for (int r = nchunk * CH; r < R; ++r) {
-                    Round x = load_round(wp, r);
-                    eat(smem, x, runp, runq, acc);
+                    for (int i = 0; i < RING; ++i)
+                        if (i >= R0 && i < R) buf[i] = load_round(wp, i);
                 }
             }
-            // ragged tail: at most one round each of 8, 4, 2 (and 1) bytes per lane
-            const int rem = p.n_lane - R * E16;
+            // ragged tail, requested now and eaten last: at most one round each of 8, 4, 2 (and 1) bytes per lane
+            uint2 t8p = make_uint2(0, 0), t8q = make_uint2(0, 0);
+            u32 t4p = 0, t4q = 0, t2p = 0, t2q = 0, t1p = 0, t1q = 0;
             if (rem) {
                 const uint8_t *t = tb + HDR + (size_t)R * 2048;
                 if (rem & (8 / ESZ)) {
-                    uint2 vp = reinterpret_cast<const uint2 *>(t)[lane], vq = reinterpret_cast<const uint2 *>(t + 512)[lane];
-                    consume<Act, MT, MODE, PRE, false, 4>(smem, vp.x, runp, acc);
-                    consume<Act, MT, MODE, PRE, false, 4>(smem, vp.y, runp, acc);
-                    consume<Act, MT, MODE, PRE, true, 4>(smem, vq.x, runq, acc);
-                    consume<Act, MT, MODE, PRE, true, 4>(smem, vq.y, runq, acc);
+                    t8p = reinterpret_cast<const uint2 *>(t)[lane];
+                    t8q = reinterpret_cast<const uint2 *>(t + 512)[lane];
                     t += 1024;
                 }
                 if (rem & (4 / ESZ)) {
-                    u32 vp = reinterpret_cast<const u32 *>(t)[lane], vq = reinterpret_cast<const u32 *>(t + 256)[lane];
-                    consume<Act, MT, MODE, PRE, false, 4>(smem, vp, runp, acc);
-                    consume<Act, MT, MODE, PRE, true, 4>(smem, vq, runq, acc);
+                    t4p = reinterpret_cast<const u32 *>(t)[lane];
+                    t4q = reinterpret_cast<const u32 *>(t + 256)[lane];
                     t += 512;
                 }
                 if (rem & (2 / ESZ)) {
-                    u32 vp = reinterpret_cast<const unsigned short *>(t)[lane], vq = reinterpret_cast<const unsigned short *>(t + 128)[lane];
-                    consume<Act, MT, MODE, PRE, false, 2>(smem, vp, runp, acc);
-                    consume<Act, MT, MODE, PRE, true, 2>(smem, vq, runq, acc);
+                    t2p = reinterpret_cast<const unsigned short *>(t)[lane];
+                    t2q = reinterpret_cast<const unsigned short *>(t + 128)[lane];
                     t += 256;
                 }
-                if constexpr (MODE == 1) {
+                if constexpr (ESZ == 1) {
                     if (rem & 1) {
-                        u32 vp = t[lane], vq = t[64 + lane];
-                        consume<Act, MT, MODE, PRE, false, 1>(smem, vp, runp, acc);
-                        consume<Act, MT, MODE, PRE, true, 1>(smem, vq, runq, acc);
+                        t1p = t[lane];
+                        t1q = t[64 + lane];
+                    }
+                }
+            }
+            if constexpr (RF == 0) {
+                int base = 0;
+                for (; base + 2 * RING <= R; base += RING) {  // steady state: eat a round, refill its slot RING rounds ahead
+#pragma unroll
+                    for (int i = 0; i < RING; ++i) {
+                        eat(smem, buf[i], runp, runq, acc);
+                        buf[i] = load_round(wp, base + RING + i);
+                    }
+                }
+                if (R - base > RING) {
+#pragma unroll
+                    for (int i = 0; i < RING; ++i) {
+                        eat(smem, buf[i], runp, runq, acc);
+                        const int r = base + RING + i;
+                        buf[i] = load_round(wp, r < R ? r : R - 1);
+                    }
+                    base += RING;
+                }
+#pragma unroll
+                for (int i = 0; i < RING; ++i) {
+                    if (base + i < R) eat(smem, buf[i], runp, runq, acc);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RF; ++i) eat(smem, buf[i], runp, runq, acc);
+            }
+            if (rem) {
+                if (rem & (8 / ESZ)) {
+                    consume<Act, MT, MODE, PRE, false, 4>(smem, t8p.x, runp, acc);
+                    consume<Act, MT, MODE, PRE, false, 4>(smem, t8p.y, runp, acc);
+                    consume<Act, MT, MODE, PRE, true, 4>(smem, t8q.x, runq, acc);
+                    consume<Act, MT, MODE, PRE, true, 4>(smem, t8q.y, runq, acc);
+                }
+                if (rem & (4 / ESZ)) {
+                    consume<Act, MT, MODE, PRE, false, 4>(smem, t4p, runp, acc);
+                    consume<Act, MT, MODE, PRE, true, 4>(smem, t4q, runq, acc);
+                }
+                if (rem & (2 / ESZ)) {
+                    consume<Act, MT, MODE, PRE, false, 2>(smem, t2p, runp, acc);
+                    consume<Act, MT, MODE, PRE, true, 2>(smem, t2q, runq, acc);
+                }
+                if constexpr (ESZ == 1) {
+                    if (rem & 1) {
+                        consume<Act, MT, MODE, PRE, false, 1>(smem, t1p, runp, acc);
+                        consume<Act, MT, MODE, PRE, true, 1>(smem, t1q, runq, acc);
                     }
                 }
             }
@@ -456,26 +478,13 @@ struct ListsBody {
 // One task = one wavefront's share of the stream: 64/L columns x L lanes, or one
 // 64-lane part of a column.  A workgroup stages the activation tile once and its
 // wavefronts then walk tasks blockIdx.x*waves + wave, + gridDim.x*waves, ...
-// blockIdx.y selects the tile of MT activation rows.  FIXED kernels carry the
-// straight-line bodies for tasks of 1, 2, 3, 4, 6 or 8 rounds; other sizes (and
-// all kernels built without FIXED) take the chunked loop.
-template <typename Act, int MT, int MODE, bool PRE, bool FIXED>
+// blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
+// exactly RF full rounds (straight-line body); RF == 0: any length (ring).
+template <typename Act, int MT, int MODE, bool PRE, int RF>
 __global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    typedef ListsBody<Act, MT, MODE, PRE> B;
-    if constexpr (FIXED) {
-        switch (p.n_lane / B::E16) {
-        case 1: B::template run<1>(p, smem); return;
-        case 2: B::template run<2>(p, smem); return;
-        case 3: B::template run<3>(p, smem); return;
-        case 4: B::template run<4>(p, smem); return;
-        case 6: B::template run<6>(p, smem); return;
-        case 8: B::template run<8>(p, smem); return;
-        default: break;
-        }
-    }
-    B::template run<0>(p, smem);
+    ListsBody<Act, MT, MODE, PRE>::template run<RF>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -487,144 +496,24 @@ struct BatchPtrs {
     void *C[BATCH_MAX];
 };
 
-template <typename Act, int MT, int MODE, bool PRE, bool FIXED>
+template <typename Act, int MT, int MODE, bool PRE, int RF>
 __global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel_batched(ListParams p, BatchPtrs b)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    typedef ListsBody<Act, MT, MODE, PRE> B;
     p.w = b.w[blockIdx.z];
     p.X = b.X[blockIdx.z];
     p.C = b.C[blockIdx.z];
-    if constexpr (FIXED) {
-        switch (p.n_lane / B::E16) {
-        case 1: B::template run<1>(p, smem); return;
-        case 2: B::template run<2>(p, smem); return;
-        case 3: B::template run<3>(p, smem); return;
-        case 4: B::template run<4>(p, smem); return;
-        case 6: B::template run<6>(p, smem); return;
-        case 8: B::template run<8>(p, smem); return;
-        default: break;
-        }
-    }
-    B::template run<0>(p, smem);
-}
-
-// ------------------------------------------------------------------- i2s GEMV
-struct I2sParams {
-    const uint4 *w;
-    const int8_t *X;
-    int *C;
-    int M, K, Kp, N, rounds;
-};
-
-// Workgroup = 16 columns; wavefront `wave` takes rounds wave, wave+waves, ...;
-// in a round lane (col%16)*4 + q reads 64 weights (rows 256*r + 64*q ...) of its column.
-// Codes 1..3 are used as they are in dot4; the "-2" of the decode
-// (bitnet_kernels.cuh:70) becomes one subtraction of 2*sum(X row) at the end.
-template <int MT>
-__global__ void __launch_bounds__(1024) i2s_kernel(I2sParams p)
-{
-    extern __shared__ __align__(16) unsigned char smem[];
-    int8_t *lx = reinterpret_cast<int8_t *>(smem);                       // [MT][Kp]
-    int *part = reinterpret_cast<int *>(smem + (size_t)MT * p.Kp);      // [waves][16][MT]
-    int *sums = part + (blockDim.x >> 6) * 16 * MT;                      // [waves][MT]
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
-    const int grp = blockIdx.x, m0 = blockIdx.y * MT;
-    constexpr int RPB = 4;
-
-    uint4 wv[RPB];
-#pragma unroll
-    for (int i = 0; i < RPB; ++i) {
-        int r = wave + i * waves;
-        wv[i] = (r < p.rounds) ? p.w[((size_t)grp * p.rounds + r) * 64 + lane] : make_uint4(0, 0, 0, 0);
-    }
-
-    // stage X rows (zero beyond M and beyond K) and accumulate the row sums on the way
-    int rs[MT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        rs[m] = 0;
-        const uint4 *src = reinterpret_cast<const uint4 *>(p.X + (size_t)(m0 + m) * p.K);
-        uint4 *dst = reinterpret_cast<uint4 *>(lx + (size_t)m * p.Kp);
-        for (int i = tid; i < p.Kp / 16; i += blockDim.x) {
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m0 + m < p.M && i < p.K / 16) v = src[i];
-            dst[i] = v;
-            rs[m] = __builtin_amdgcn_sdot4((int)v.x, 0x01010101, rs[m], false);
-            rs[m] = __builtin_amdgcn_sdot4((int)v.y, 0x01010101, rs[m], false);
-            rs[m] = __builtin_amdgcn_sdot4((int)v.z, 0x01010101, rs[m], false);
-            rs[m] = __builtin_amdgcn_sdot4((int)v.w, 0x01010101, rs[m], false);
-        }
-        rs[m] = lanes_sum(rs[m], 6);
-        if (lane == 0) sums[wave * MT + m] = rs[m];
-    }
-    __syncthreads();
-
-    int acc[MT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = 0;
-    const int q = lane & 3;
-
-    for (int r0 = wave;; r0 += RPB * waves) {
-#pragma unroll
-        for (int i = 0; i < RPB; ++i) {
-            const int r = r0 + i * waves;
-            if (r < p.rounds) {
-                const u32 words[4] = {wv[i].x, wv[i].y, wv[i].z, wv[i].w};
-#pragma unroll
-                for (int m = 0; m < MT; ++m) {
-                    const uint4 *xr = reinterpret_cast<const uint4 *>(lx + (size_t)m * p.Kp + 256 * r + 64 * q);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint4 x = xr[j];
-                        const u32 wd = words[j];
-                        acc[m] = __builtin_amdgcn_sdot4((int)x.x, (int)(wd & 0x03030303u), acc[m], false);
-                        acc[m] = __builtin_amdgcn_sdot4((int)x.y, (int)((wd >> 2) & 0x03030303u), acc[m], false);
-                        acc[m] = __builtin_amdgcn_sdot4((int)x.z, (int)((wd >> 4) & 0x03030303u), acc[m], false);
-                        acc[m] = __builtin_amdgcn_sdot4((int)x.w, (int)((wd >> 6) & 0x03030303u), acc[m], false);
-                    }
-                }
-            }
-        }
-        if (r0 + RPB * waves >= p.rounds) break;
-#pragma unroll
-        for (int i = 0; i < RPB; ++i) {
-            int r = r0 + (RPB + i) * waves;
-            wv[i] = (r < p.rounds) ? p.w[((size_t)grp * p.rounds + r) * 64 + lane] : make_uint4(0, 0, 0, 0);
-        }
-    }
-
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        acc[m] = lanes_sum(acc[m], 2);
-        if (q == 0) part[(wave * 16 + (lane >> 2)) * MT + m] = acc[m];
-    }
-    __syncthreads();
-    for (int t = tid; t < 16 * MT; t += blockDim.x) {
-        const int col = t / MT, m = t % MT;
-        int s = 0, sx = 0;
-        for (int w = 0; w < waves; ++w) {
-            s += part[(w * 16 + col) * MT + m];
-            sx += sums[w * MT + m];
-        }
-        if (m0 + m < p.M) p.C[(size_t)(m0 + m) * p.N + grp * 16 + col] = s - 2 * sx;
-    }
-}
-
-__global__ void __launch_bounds__(256) copy_kernel(uint4 *dst, const uint4 *src, size_t n16)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+    ListsBody<Act, MT, MODE, PRE>::template run<RF>(p, smem);
 }
 
 // ------------------------------------------------------------------ launchers
-static int hip_fail(hipError_t e, const char *what)
+static inline int hip_fail(hipError_t e, const char *what)
 {
     return fail(SPTMM_ERR_HIP, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
 }
 
 // Dynamic LDS above the default cap has to be granted per kernel once.
-static int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &granted)
+static inline int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &granted)
 {
     if (lds <= granted.load(std::memory_order_relaxed)) return SPTMM_OK;
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -633,8 +522,8 @@ static int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &granted)
     return SPTMM_OK;
 }
 
-template <typename Act, int MT, int MODE, bool PRE>
-static int launch_lists_t(const GemvArgs &a, hipStream_t st)
+template <typename Act, int MT, int MODE, bool PRE, int RF>
+static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
 {
     // Wavefronts per workgroup: fill the CUs with one workgroup each, and when a
     // CU gets more than LISTS_MAX_WAVES tasks pick the count that wastes the
@@ -658,16 +547,15 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
     const int blocks = (a.tasks + wpb - 1) / wpb;
     const int grid_x = blocks < slots ? blocks : slots;
     const int iters = (blocks + grid_x - 1) / grid_x;
-    ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, a.n_lane, a.tasks, ilog2(a.L), a.W, iters};
+    ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, MODE == 3 ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
+                 a.task_stride, iters};
     constexpr int SLOT = slot_bytes<Act, MT>();
-    size_t lds = (((size_t)(a.K + 1) * SLOT + 15) & ~(size_t)15) + (size_t)wpb * MT * sizeof(typename Acc<Act>::type);
+    size_t lds = (size_t)(a.K + 64) * SLOT + (size_t)wpb * MT * sizeof(typename Acc<Act>::type);
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
-    // straight-line bodies for the int8 paths of the u16 and 8-bit gap streams
-    constexpr bool FIXED = sizeof(Act) == 1 && MODE != 2;
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     if (a.batch) {
         if constexpr (sizeof(Act) == 1) {
-            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, FIXED>;
+            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, RF>;
             static std::atomic<size_t> lds_granted_b{48 * 1024};
             if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_b)) return rc;
             for (int first = 0; first < a.batch; first += BATCH_MAX) {
@@ -688,7 +576,7 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
             return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take int8 activations");
         }
     }
-    auto kern = lists_kernel<Act, MT, MODE, PRE, FIXED>;
+    auto kern = lists_kernel<Act, MT, MODE, PRE, RF>;
     static std::atomic<size_t> lds_granted{48 * 1024};
     if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
     hipLaunchKernelGGL(kern, grid, block, lds, st, p);
@@ -696,14 +584,33 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel launch");
 }
 
+// Straight-line bodies exist for the int8 paths of the u16 and 8-bit run streams
+// with 1, 2, 3, 4, 6 or 8 full rounds per task; everything else takes the ring.
+template <typename Act, int MT, int MODE, bool PRE>
+static int launch_lists_t(const GemvArgs &a, hipStream_t st)
+{
+    if constexpr (sizeof(Act) == 1 && MODE < 2) {
+        switch (a.n_lane / (MODE == 1 ? 16 : 8)) {
+        case 1: return launch_lists_rf<Act, MT, MODE, PRE, 1>(a, st);
+        case 2: return launch_lists_rf<Act, MT, MODE, PRE, 2>(a, st);
+        case 3: return launch_lists_rf<Act, MT, MODE, PRE, 3>(a, st);
+        case 4: return launch_lists_rf<Act, MT, MODE, PRE, 4>(a, st);
+        case 6: return launch_lists_rf<Act, MT, MODE, PRE, 6>(a, st);
+        case 8: return launch_lists_rf<Act, MT, MODE, PRE, 8>(a, st);
+        default: break;
+        }
+    }
+    return launch_lists_rf<Act, MT, MODE, PRE, 0>(a, st);
+}
+
 template <typename Act, int MODE, bool PRE>
 static int launch_lists_m(const GemvArgs &a, hipStream_t st)
 {
     const size_t lim = (size_t)a.lds_limit - 256;
     if constexpr (sizeof(Act) == 1) {
-        if (a.M >= 5 && (size_t)(a.K + 1) * slot_bytes<Act, 8>() <= lim) return launch_lists_t<Act, 8, MODE, PRE>(a, st);
+        if (a.M >= 5 && (size_t)(a.K + 64) * slot_bytes<Act, 8>() <= lim) return launch_lists_t<Act, 8, MODE, PRE>(a, st);
     }
-    if (a.M >= 2 && (size_t)(a.K + 1) * slot_bytes<Act, 4>() <= lim) return launch_lists_t<Act, 4, MODE, PRE>(a, st);
+    if (a.M >= 2 && (size_t)(a.K + 64) * slot_bytes<Act, 4>() <= lim) return launch_lists_t<Act, 4, MODE, PRE>(a, st);
     return launch_lists_t<Act, 1, MODE, PRE>(a, st);
 }
 
@@ -716,58 +623,6 @@ static int launch_lists_a(const GemvArgs &a, ActType act, hipStream_t st)
     case ACT_F32: return launch_lists_m<float, MODE, PRE>(a, st);
     }
     return fail(SPTMM_ERR_INVALID, "unknown activation type");
-}
-
-int launch_u16(const GemvArgs &a, ActType act, void *stream)
-{
-    if (a.index_shift == 2) return launch_lists_a<0, true>(a, act, (hipStream_t)stream);
-    return launch_lists_a<0, false>(a, act, (hipStream_t)stream);
-}
-
-int launch_delta(const GemvArgs &a, ActType act, void *stream)
-{
-    if (a.delta_bits == 8) return launch_lists_a<1, false>(a, act, (hipStream_t)stream);
-    return launch_lists_a<2, false>(a, act, (hipStream_t)stream);
-}
-
-template <int MT>
-static int launch_i2s_t(const GemvArgs &a, hipStream_t st, int waves)
-{
-    const int Kp = i2s_padded_k(a.K);
-    I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256};
-    size_t lds = (size_t)MT * Kp + (size_t)waves * 16 * MT * 4 + (size_t)waves * MT * 4;
-    auto kern = i2s_kernel<MT>;
-    static std::atomic<size_t> lds_granted{48 * 1024};
-    if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
-    dim3 grid(a.N / 16, (a.M + MT - 1) / MT), block(64 * waves);
-    hipLaunchKernelGGL(kern, grid, block, lds, st, p);
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? SPTMM_OK : hip_fail(e, "i2s_kernel launch");
-}
-
-int launch_i2s(const GemvArgs &a, void *stream)
-{
-    const int Kp = i2s_padded_k(a.K), rounds = Kp / 256, groups = a.N / 16;
-    int rpw = groups >= 2 * a.compute_units ? 4 : (groups >= a.compute_units ? 2 : 1);
-    int waves = (rounds + rpw - 1) / rpw;
-    waves = waves < 1 ? 1 : (waves > 16 ? 16 : waves);
-    const size_t extra = (size_t)waves * 17 * 4;
-    hipStream_t st = (hipStream_t)stream;
-    if (a.M >= 5 && (size_t)8 * Kp + extra * 8 <= (size_t)a.lds_limit) return launch_i2s_t<8>(a, st, waves);
-    if (a.M >= 2 && (size_t)4 * Kp + extra * 4 <= (size_t)a.lds_limit) return launch_i2s_t<4>(a, st, waves);
-    if ((size_t)Kp + extra > (size_t)a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "K too large for the LDS activation tile");
-    return launch_i2s_t<1>(a, st, waves);
-}
-
-int launch_copy(void *dst, const void *src, size_t bytes, void *stream)
-{
-    if (bytes % 16) return fail(SPTMM_ERR_INVALID, "copy size must be a multiple of 16 bytes");
-    size_t n16 = bytes / 16;
-    int blocks = (int)((n16 + 255) / 256 < 256 * 64 ? (n16 + 255) / 256 : 256 * 64);
-    if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint4 *)dst, (const uint4 *)src, n16);
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? SPTMM_OK : hip_fail(e, "copy_kernel launch");
 }
 
 }  // namespace sptmm

@@ -1,0 +1,108 @@
+"""Timing sweeps over the benchmark's other shapes, all three encodings of the same seeded matrix.
+
+    python -m sptmm_amd.sweep layer     # BitNet-b1.58-2B decoder layer: q/o, k/v, gate/up (K=2560), down (K=6912)
+    python -m sptmm_amd.sweep large     # K=13824 N=5120 S=8320, M in {1, 8, 16}
+    python -m sptmm_amd.sweep headline  # K=6912 N=2560 S=4096, M in {1, 4}
+
+Per shape and encoding: microseconds per GEMV launched alone (cache-warm = the same stream every launch;
+HBM-cold = rotating over enough device copies to exceed the 256 MB last-level cache) and, for the list
+encodings, per GEMV inside one batched launch.  Every timed object is first checked against the other
+encodings (bit-exact int32).  Prints a table and one JSON line.
+"""
+from __future__ import annotations
+
+import json
+import sys
+
+import numpy as np
+
+from . import _capi as sp
+
+PEAK_GBPS = 8000.0
+LAYER = [("q/o", 2560, 2560, 1536, 2), ("k/v", 2560, 640, 1536, 2), ("gate/up", 2560, 6912, 1536, 2),
+         ("down", 6912, 2560, 4160, 1)]
+
+
+def copies_for(nbytes: int) -> int:
+    return max(2, min(64, int(np.ceil(640e6 / nbytes))))
+
+
+def time_weights(w, X, M, N, st, batched: bool):
+    xb = sp.DeviceBuffer.from_numpy(X)
+    n = copies_for(w.nbytes)
+    cps = [w] + [w.clone() for _ in range(n - 1)]
+    cb = sp.DeviceBuffer(4 * M * N * min(n, 32))
+    sp.measure_gemv(cps[:1], 0, xb, M, cb, 200, 0, st)
+    warm = min(sp.measure_gemv(cps[:1], 0, xb, M, cb, 2000, 0, st) for _ in range(3))
+    sp.measure_gemv(cps, 0, xb, M, cb, 2 * n, 0, st)
+    cold = min(sp.measure_gemv(cps, 0, xb, M, cb, 2000, 0, st) for _ in range(3))
+    bat = None
+    if batched:
+        nb = min(n, 32)
+        sp.measure_gemv(cps[:nb], 0, xb, M, cb, 4 * nb, 3, st)
+        bat = min(sp.measure_gemv(cps[:nb], 0, xb, M, cb, 64 * nb, 3, st) for _ in range(3))
+    for c in cps[1:]:
+        c.free()
+    xb.free()
+    cb.free()
+    return warm, cold, bat
+
+
+def run_shape(name, K, N, S, Ms, splits, st, rows):
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    for M in Ms:
+        X = sp.make_x_i8(0xC0FFEE ^ M, M, K)
+        ref = None
+        cands = [("u16/%d" % s, lambda s=s: sp.Weights.upload_u16(pos, neg, K, s)) for s in splits if (S // 2) % s == 0]
+        cands += [("delta/%d" % s, lambda s=s: sp.Weights.upload_delta(pos, neg, K, s)) for s in splits
+                  if s <= 64 and (S // 2) % s == 0]
+        cands += [("i2s", lambda: sp.Weights.upload_i2s(W))]
+        for enc, mk in cands:
+            w = mk()
+            got = w.matmul(X)
+            if ref is None:
+                ref = got
+            ok = bool((got == ref).all())
+            nbytes = w.nbytes + M * K + 4 * M * N
+            warm, cold, bat = time_weights(w, X, M, N, st, enc != "i2s")
+            w.free()
+            rows.append({"shape": name, "K": K, "N": N, "S": S, "M": M, "enc": enc, "bytes": nbytes, "ok": ok,
+                         "warm_us": round(warm, 3), "cold_us": round(cold, 3),
+                         "batched_us": None if bat is None else round(bat, 3)})
+            r = rows[-1]
+            print("%-8s K=%-5d N=%-5d S=%-5d M=%-2d %-9s %s  warm %7.2f us  cold %7.2f us (%5.0f GB/s)  batched %s"
+                  % (name, K, N, S, M, enc, "ok " if ok else "BAD", warm, cold, nbytes / cold / 1e3,
+                     "   -   " if bat is None else "%7.2f us (%5.0f GB/s, %4.1f%%)" % (bat, nbytes / bat / 1e3,
+                                                                                     nbytes / bat / 1e3 / PEAK_GBPS * 100)),
+                  flush=True)
+
+
+def main(argv):
+    which = argv[1] if len(argv) > 1 else "layer"
+    info = sp.device_init(0)
+    st = sp.Stream()
+    rows = []
+    if which == "layer":
+        for name, K, N, S, _ in LAYER:
+            run_shape(name, K, N, S, (1, 4), (8, 16, 32, 64), st, rows)
+        for M in (1, 4):
+            for kind in ("u16", "delta", "i2s"):
+                tot_w = tot_c = 0.0
+                for name, K, N, S, mult in LAYER:
+                    best = [r for r in rows if r["shape"] == name and r["M"] == M and r["enc"].startswith(kind)]
+                    tot_w += mult * min(r["warm_us"] for r in best)
+                    tot_c += mult * min(r["cold_us"] for r in best)
+                print("layer sum (7 GEMVs, best split per shape) M=%d %-5s: warm %.1f us  cold %.1f us" % (M, kind, tot_w, tot_c))
+                rows.append({"shape": "layer_sum", "M": M, "enc": kind, "warm_us": round(tot_w, 2), "cold_us": round(tot_c, 2)})
+    elif which == "large":
+        run_shape("large", 13824, 5120, 8320, (1, 8, 16), (32, 64), st, rows)
+    elif which == "headline":
+        run_shape("headline", 6912, 2560, 4096, (1, 4), (16, 32, 64), st, rows)
+    else:
+        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline")
+    assert all(r.get("ok", True) for r in rows), "encodings disagree"
+    print(json.dumps({"device": info["arch"], "rows": rows}))
+
+
+if __name__ == "__main__":
+    main(sys.argv)
