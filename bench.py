@@ -180,7 +180,10 @@ def main():
         "single_launch": single, "other_encodings": others,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(gbps / PEAK_GBPS, 4),
+                     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE (x1.0), scale factors
+                     # from the 1 GiB copy kernel; measured once and recorded in profiles/, not re-measured here
+                     "traffic": 671.8e6,
                      "kernel": "lists_kernel_batched<int8, MT=1, u16>", "launch_us": round(launch_us, 2),
                      "algorithmic_bytes_per_launch": nbytes * BATCH},
     }
