@@ -56,8 +56,9 @@ typedef struct sptmm_winfo {
     int K, N, S;     /* S = nonzeros per column (0 for i2s) */
     int split_k;     /* lanes cooperating on one column (0 for i2s) */
     int delta_bits;  /* 8 or 16 for SPTMM_KIND_DELTA, else 0 */
-    int delta_layout; /* SPTMM_KIND_DELTA: 1 = contiguous runs, 2 = striped by row mod 32; else 0 */
     uint64_t stream_bytes; /* bytes of the weight stream one GEMV reads */
+    int ragged;      /* 1: built from a matrix whose columns differ in nonzeros (S is 0 then) */
+    uint64_t nnz;    /* nonzeros of the whole matrix */
 } sptmm_winfo;
 
 typedef struct sptmm_weights sptmm_weights; /* opaque; owns its device buffer */
@@ -99,21 +100,28 @@ size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits);
 int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out);
 int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg);
 
-/* Striped gap stream, split_k 32 or 64: lane v of a column owns the rows of one
- * residue class mod 32 (row = v%32 + 32*j) and stores the gaps of j as bytes, so
- * the 32 lanes of a half-wavefront always read 32 different LDS banks; the
- * lists of a wavefront are padded to a common length with entries that land on
- * zero rows behind the activation tile.  Costs ~30 % more bytes (and 1.5x the
- * gathers) than the run layout above and removes its bank conflicts; measured
- * slower than runs on MI355X, so uploads use it only on request.  _eligible returns 1 when every
- * gap (in units of 32 rows) fits a byte, 0 when not, < 0 on bad arguments.
- * _bytes returns the size of the stream (0 if not eligible); *read_bytes is
- * what one GEMV reads of it (tasks are stored at a fixed stride). */
-int sptmm_delta_striped_eligible(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k);
-size_t sptmm_pack_delta_striped_bytes(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k,
-                                      size_t *read_bytes, int *n_min, int *n_max);
-int sptmm_pack_delta_striped(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out);
-int sptmm_unpack_delta_striped(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg);
+/* Ragged matrices: any K x N matrix over {-1,0,+1} (column n at W + n*K), columns
+ * free to differ in nonzeros and in their +1/-1 split -- what a quantised model
+ * tensor looks like.  No counterpart in the reference, whose generator and
+ * kernels fix S/2 entries per sign and column (main.cu:90, 276, 564); its unused
+ * "VCSC" arrays (main.cu:461-488) sketch per-column counts.  kind is
+ * SPTMM_KIND_U16 (split_k 8..256) or SPTMM_KIND_DELTA (split_k 8..64).  The
+ * stream opens with one entry count per wavefront task; a task pads its shorter
+ * lists with entries on the zero rows K..K+63 that the activation tile keeps;
+ * K + 64 must fit 16 bits.  *bits (gap streams): in 0 = pick 8 when every gap fits a byte,
+ * else 16; out the width used.  _bytes returns the stream size (0 on error);
+ * *read_bytes is what one GEMV reads of it (tasks sit at a fixed stride). */
+size_t sptmm_pack_ragged_bytes(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int *bits, size_t *read_bytes,
+                               int *n_min, int *n_max, uint64_t *nnz);
+int sptmm_pack_ragged(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int bits, void *out);
+int sptmm_unpack_ragged(const void *packed, int K, int N, int kind, int split_k, int bits, int8_t *W_colmajor);
+/* Seeded matrix with independent entries: +1 with probability p_pos, -1 with
+ * p_neg (xorshift32 of macro.cuh:69-76 per column, state seed ^ 0x9E3779B9*(n+1);
+ * entry = top 24 bits of the next state against the two thresholds). */
+int sptmm_generate_ternary_iid(int K, int N, uint32_t seed, double p_pos, double p_neg, int8_t *W_colmajor);
+/* Dense matrix from 2-bit words in the reference's own order: word g of column n
+ * at words[n*(K/16) + g] holds rows 16g..16g+15 (main.cu:176-196). */
+int sptmm_dense_from_i2s_words(const uint32_t *words, int K, int N, int8_t *W_colmajor);
 
 /* i2s: 16 weights per word, code = w + 2, element e at bit 8*(e%4) + 2*(e/4)
  * (main.cu:176-192, decode bitnet_kernels.cuh:52-72).  Word order is this
@@ -134,10 +142,11 @@ int sptmm_device_init(int device, sptmm_devinfo *out);
  * prepareW_map / prepareW_i2s sequence of main.cu:914-989 and 1851-1859. */
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
-/* layout: 0 = default (runs), 1 = runs, 2 = striped (kept as an alternative; slower where measured) */
-int sptmm_weights_upload_delta_layout(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int layout,
-                                      sptmm_weights **out);
 int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weights **out);
+/* Any ternary matrix -> device stream of the given kind (ragged u16 lists,
+ * ragged gap stream, or i2s).  The GEMV entry points below serve it like any
+ * other weights object. */
+int sptmm_weights_upload_dense(const int8_t *W_colmajor, int K, int N, int kind, int split_k, sptmm_weights **out);
 /* Second device copy of the same stream (used to rotate over more bytes than
  * the last-level cache holds when timing cold reads). */
 int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out);

@@ -8,8 +8,8 @@ import numpy as np
 
 __all__ = [
     "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
-    "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "delta_striped_eligible",
-    "pack_delta_striped", "unpack_delta_striped", "pack_i2s", "unpack_i2s",
+    "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
+    "generate_ternary_iid", "dense_from_i2s_words",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel",
     "device_sync", "measure_gemv", "gemv_i8_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
@@ -22,10 +22,11 @@ _LIB = None
 EXPORTS = [
     "sptmm_last_error", "sptmm_version", "sptmm_generate_ternary", "sptmm_lists_from_dense", "sptmm_make_x_i8",
     "sptmm_pack_u16_bytes", "sptmm_pack_u16", "sptmm_unpack_u16", "sptmm_delta_bits", "sptmm_pack_delta_bytes",
-    "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_delta_striped_eligible", "sptmm_pack_delta_striped_bytes",
-    "sptmm_pack_delta_striped", "sptmm_unpack_delta_striped", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
-    "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_device_init",
-    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_delta_layout",
+    "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
+    "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_pack_ragged_bytes", "sptmm_pack_ragged",
+    "sptmm_unpack_ragged", "sptmm_generate_ternary_iid", "sptmm_dense_from_i2s_words", "sptmm_weights_upload_dense",
+    "sptmm_device_init",
+    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
     "sptmm_gemv_f32", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
@@ -49,7 +50,8 @@ class DevInfo(C.Structure):
 
 class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
-                ("delta_bits", C.c_int), ("delta_layout", C.c_int), ("stream_bytes", C.c_uint64)]
+                ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64),
+                ("ragged", C.c_int), ("nnz", C.c_uint64)]
 
 
 def lib_path() -> str:
@@ -68,7 +70,7 @@ def lib() -> C.CDLL:
         L.sptmm_last_error.restype = C.c_char_p
         L.sptmm_version.restype = C.c_char_p
         for n in ("sptmm_pack_u16_bytes", "sptmm_pack_delta_bytes", "sptmm_pack_i2s_bytes", "sptmm_weights_bytes",
-                  "sptmm_pack_delta_striped_bytes"):
+                  "sptmm_pack_ragged_bytes"):
             getattr(L, n).restype = C.c_size_t
         L.sptmm_i2s_pack_word.restype = C.c_uint32
         L.sptmm_i2s_decode_word.restype = None
@@ -89,6 +91,7 @@ def lib() -> C.CDLL:
                                          C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         L.sptmm_copy_kernel.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         L.sptmm_make_x_i8.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p]
+        L.sptmm_generate_ternary_iid.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_double, C.c_double, C.c_void_p]
         for n in ("sptmm_stream_create", "sptmm_event_create"):
             getattr(L, n).argtypes = [C.POINTER(C.c_void_p)]
         for n in ("sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_event_destroy", "sptmm_event_sync"):
@@ -181,30 +184,6 @@ def unpack_delta(packed, K, N, S, split_k, bits):
     return pos, neg
 
 
-def delta_striped_eligible(pos, neg, K, split_k) -> bool:
-    N, half = pos.shape
-    return bool(_ck(lib().sptmm_delta_striped_eligible(_p(pos), _p(neg), K, N, 2 * half, split_k)))
-
-
-def pack_delta_striped(pos, neg, K, split_k):
-    """-> (stream bytes, dict(read_bytes, n_min, n_max))."""
-    N, half = pos.shape
-    rb, lo, hi = C.c_size_t(), C.c_int(), C.c_int()
-    n = lib().sptmm_pack_delta_striped_bytes(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(rb), C.byref(lo), C.byref(hi))
-    if not n:
-        raise SptmmError(-2, "matrix not eligible for the striped gap layout")
-    out = np.zeros(n, np.uint8)
-    _ck(lib().sptmm_pack_delta_striped(_p(pos), _p(neg), K, N, 2 * half, split_k, _p(out)))
-    return out, {"read_bytes": rb.value, "n_min": lo.value, "n_max": hi.value}
-
-
-def unpack_delta_striped(packed, K, N, S, split_k):
-    pos = np.empty((N, S // 2), np.uint16)
-    neg = np.empty((N, S // 2), np.uint16)
-    _ck(lib().sptmm_unpack_delta_striped(_p(packed), K, N, S, split_k, _p(pos), _p(neg)))
-    return pos, neg
-
-
 def i2s_pack_word(w16) -> int:
     a = np.ascontiguousarray(w16, np.int8)
     assert a.size == 16
@@ -228,6 +207,39 @@ def pack_i2s(W: np.ndarray) -> np.ndarray:
 def unpack_i2s(packed, K, N) -> np.ndarray:
     W = np.empty((N, K), np.int8)
     _ck(lib().sptmm_unpack_i2s(_p(packed), K, N, _p(W)))
+    return W
+
+
+def generate_ternary_iid(K: int, N: int, seed: int, p_pos: float, p_neg: float) -> np.ndarray:
+    """-> W [N][K] int8 (column-major K x N) with independent entries."""
+    W = np.empty((max(N, 0), max(K, 0)), np.int8)
+    _ck(lib().sptmm_generate_ternary_iid(K, N, seed & 0xFFFFFFFF, p_pos, p_neg, _p(W)))
+    return W
+
+
+def dense_from_i2s_words(words: np.ndarray, K: int) -> np.ndarray:
+    """words [N][K/16] u32 in the reference's order -> W [N][K] int8."""
+    N = words.shape[0]
+    W = np.empty((N, K), np.int8)
+    _ck(lib().sptmm_dense_from_i2s_words(_p(np.ascontiguousarray(words, np.uint32)), K, N, _p(W)))
+    return W
+
+
+def pack_ragged(W: np.ndarray, kind: int, split_k: int, bits: int = 0):
+    """Any ternary matrix W [N][K] -> (stream bytes, dict(bits, read_bytes, n_min, n_max, nnz))."""
+    N, K = W.shape
+    b, rb, lo, hi, nnz = C.c_int(bits), C.c_size_t(), C.c_int(), C.c_int(), C.c_uint64()
+    n = lib().sptmm_pack_ragged_bytes(_p(W), K, N, kind, split_k, C.byref(b), C.byref(rb), C.byref(lo), C.byref(hi), C.byref(nnz))
+    if not n:
+        raise SptmmError(-1, lib().sptmm_last_error().decode())
+    out = np.zeros(n, np.uint8)
+    _ck(lib().sptmm_pack_ragged(_p(W), K, N, kind, split_k, b.value, _p(out)))
+    return out, {"bits": b.value, "read_bytes": rb.value, "n_min": lo.value, "n_max": hi.value, "nnz": nnz.value}
+
+
+def unpack_ragged(packed: np.ndarray, K: int, N: int, kind: int, split_k: int, bits: int = 0) -> np.ndarray:
+    W = np.empty((N, K), np.int8)
+    _ck(lib().sptmm_unpack_ragged(_p(packed), K, N, kind, split_k, bits, _p(W)))
     return W
 
 
@@ -354,11 +366,10 @@ class Weights:
         return cls(h)
 
     @classmethod
-    def upload_delta(cls, pos, neg, K, split_k, layout: int = 0) -> "Weights":
-        """layout: 0 / 1 = contiguous runs (default), 2 = striped by row mod 32 (alternative, slower where measured)."""
+    def upload_delta(cls, pos, neg, K, split_k) -> "Weights":
         N, half = pos.shape
         h = C.c_void_p()
-        _ck(lib().sptmm_weights_upload_delta_layout(_p(pos), _p(neg), K, N, 2 * half, split_k, layout, C.byref(h)))
+        _ck(lib().sptmm_weights_upload_delta(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(h)))
         return cls(h)
 
     @classmethod
@@ -366,6 +377,14 @@ class Weights:
         N, K = W.shape
         h = C.c_void_p()
         _ck(lib().sptmm_weights_upload_i2s(_p(W), K, N, C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def upload_dense(cls, W: np.ndarray, kind: int, split_k: int = 32) -> "Weights":
+        """Any ternary matrix W [N][K] (columns free to differ in nonzeros) in the given encoding."""
+        N, K = W.shape
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_upload_dense(_p(W), K, N, kind, split_k, C.byref(h)))
         return cls(h)
 
     def clone(self) -> "Weights":

@@ -19,8 +19,9 @@ struct sptmm_weights {
     int device;
     int compute_units;
     int lds_limit;
-    int task_stride = 0;  // striped gap stream
+    int task_stride = 0, counts_bytes = 0;  // ragged streams
     int n_min = 0, n_max = 0;
+    int index_shift = 0;  // u16 streams: fields are row << index_shift
 };
 
 namespace {
@@ -104,11 +105,12 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.G = w->geo.G;
     a.W = w->geo.W;
     a.delta_bits = w->info.delta_bits;
-    a.delta_layout = w->info.delta_layout;
     a.task_stride = w->task_stride;
+    a.counts_bytes = w->counts_bytes;
     a.n_min = w->n_min;
     a.n_max = w->n_max;
-    a.index_shift = w->info.kind == SPTMM_KIND_U16 ? u16_index_shift(w->info.K) : 0;
+    a.index_shift = w->index_shift;
+    a.ragged = w->info.ragged;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
     a.batch = batch;
@@ -162,53 +164,27 @@ int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, in
     if (int rc = sptmm_pack_u16(pos, neg, K, N, S, split_k, host.data())) return rc;
     sptmm_weights *w = new (std::nothrow) sptmm_weights();
     if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{SPTMM_KIND_U16, K, N, S, split_k, 0, 0, 0};
-    w->geo = g;
-    return finish_upload(w, host, out);
-}
-
-int sptmm_weights_upload_delta_layout(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int layout,
-                                      sptmm_weights **out)
-{
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (layout < 0 || layout > 2) return fail(SPTMM_ERR_INVALID, "layout must be 0 (auto), 1 (runs) or 2 (striped)");
-    if (int rc = check_shape(K, N, S)) return rc;
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
-    // Measured on MI355X (headline shape): the striped layout reads ~1.3x the bytes and runs 1.5x the
-    // gathers of the run layout; its conflict-free LDS access does not pay for that, so runs are the default.
-    if (layout == 0) layout = 1;
-    sptmm_weights *w = nullptr;
-    std::vector<uint8_t> host;
-    if (layout == 2) {
-        size_t read_bytes = 0;
-        int n_min = 0, n_max = 0;
-        size_t bytes = sptmm_pack_delta_striped_bytes(pos, neg, K, N, S, split_k, &read_bytes, &n_min, &n_max);
-        if (!bytes) return fail(SPTMM_ERR_UNSUPPORTED, "this matrix cannot take the striped gap layout (split_k 32/64, gaps of at most 255*32 rows)");
-        host.resize(bytes);
-        if (int rc = sptmm_pack_delta_striped(pos, neg, K, N, S, split_k, host.data())) return rc;
-        w = new (std::nothrow) sptmm_weights();
-        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-        w->info = sptmm_winfo{SPTMM_KIND_DELTA, K, N, S, split_k, 8, 2, read_bytes};
-        w->task_stride = 272 + 128 * n_max;
-        w->n_min = n_min;
-        w->n_max = n_max;
-    } else {
-        int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
-        if (bits < 0) return bits;
-        host.resize(sptmm_pack_delta_bytes(N, S, split_k, bits));
-        if (int rc = sptmm_pack_delta(pos, neg, K, N, S, split_k, bits, host.data())) return rc;
-        w = new (std::nothrow) sptmm_weights();
-        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-        w->info = sptmm_winfo{SPTMM_KIND_DELTA, K, N, S, split_k, bits, 1, 0};
-    }
+    w->info = sptmm_winfo{SPTMM_KIND_U16, K, N, S, split_k, 0, 0, 0, (uint64_t)S * N};
+    w->index_shift = u16_index_shift(K);
     w->geo = g;
     return finish_upload(w, host, out);
 }
 
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out)
 {
-    return sptmm_weights_upload_delta_layout(pos, neg, K, N, S, split_k, 0, out);
+    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (int rc = check_shape(K, N, S)) return rc;
+    Geometry g;
+    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
+    int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
+    if (bits < 0) return bits;
+    std::vector<uint8_t> host(sptmm_pack_delta_bytes(N, S, split_k, bits));
+    if (int rc = sptmm_pack_delta(pos, neg, K, N, S, split_k, bits, host.data())) return rc;
+    sptmm_weights *w = new (std::nothrow) sptmm_weights();
+    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+    w->info = sptmm_winfo{SPTMM_KIND_DELTA, K, N, S, split_k, bits, 0, 0, (uint64_t)S * N};
+    w->geo = g;
+    return finish_upload(w, host, out);
 }
 
 int sptmm_weights_upload_i2s(const int8_t *W, int K, int N, sptmm_weights **out)
@@ -220,8 +196,34 @@ int sptmm_weights_upload_i2s(const int8_t *W, int K, int N, sptmm_weights **out)
     if (int rc = sptmm_pack_i2s(W, K, N, host.data())) return rc;
     sptmm_weights *w = new (std::nothrow) sptmm_weights();
     if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{SPTMM_KIND_I2S, K, N, 0, 0, 0, 0, 0};
+    w->info = sptmm_winfo{SPTMM_KIND_I2S, K, N, 0, 0, 0, 0, 0, 0};
     w->geo = Geometry{};
+    return finish_upload(w, host, out);
+}
+
+int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int split_k, sptmm_weights **out)
+{
+    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (kind == SPTMM_KIND_I2S) return sptmm_weights_upload_i2s(W, K, N, out);
+    int bits = 0, n_min = 0, n_max = 0;
+    size_t read_bytes = 0;
+    uint64_t nnz = 0;
+    const size_t bytes = sptmm_pack_ragged_bytes(W, K, N, kind, split_k, &bits, &read_bytes, &n_min, &n_max, &nnz);
+    if (!bytes) return SPTMM_ERR_INVALID;  // message set by the planner
+    std::vector<uint8_t> host(bytes);
+    if (int rc = sptmm_pack_ragged(W, K, N, kind, split_k, bits, host.data())) return rc;
+    sptmm_weights *w = new (std::nothrow) sptmm_weights();
+    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+    w->info = sptmm_winfo{kind, K, N, 0, split_k, bits, read_bytes, 1, nnz};
+    if (int rc = make_ragged_geometry(N, split_k, 256, &w->geo)) {
+        delete w;
+        return rc;
+    }
+    w->counts_bytes = (int)ragged_counts_bytes(w->geo.tasks);
+    w->task_stride = (int)((bytes - w->counts_bytes) / w->geo.tasks);
+    w->n_min = n_min;
+    w->n_max = n_max;
+    w->index_shift = kind == SPTMM_KIND_U16 ? ragged_index_shift(K) : 0;
     return finish_upload(w, host, out);
 }
 
@@ -273,7 +275,8 @@ int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X
         const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
         if (b.kind == SPTMM_KIND_I2S) return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take u16 or gap streams");
         if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
-            a.delta_layout != b.delta_layout || ws[0]->task_stride != ws[i]->task_stride)
+            a.ragged != b.ragged || ws[0]->task_stride != ws[i]->task_stride ||
+            ws[0]->n_min != ws[i]->n_min)
             return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);
         wp[i] = ws[i]->dev;
         xp[i] = X[i];

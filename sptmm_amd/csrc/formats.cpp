@@ -55,6 +55,23 @@ int make_geometry(int N, int S, int split_k, int max_split, Geometry *g)
     return SPTMM_OK;
 }
 
+int make_ragged_geometry(int N, int split_k, int max_split, Geometry *g)
+{
+    bool ok = false;
+    for (int s = 8; s <= max_split; s *= 2) ok |= (s == split_k);
+    if (!ok) return fail(SPTMM_ERR_INVALID, "Wrong split size");
+    g->N = N;
+    g->half = 0;
+    g->split_k = split_k;
+    g->L = std::min(split_k, 64);
+    g->G = 64 / g->L;
+    g->W = std::max(1, split_k / 64);
+    g->n_lane = 0;
+    if (N % g->G) return fail(SPTMM_ERR_INVALID, "N must be a multiple of %d for split_k=%d", g->G, split_k);
+    g->tasks = N / g->G * g->W;
+    return SPTMM_OK;
+}
+
 size_t slot_offset(int n_lane, int esz, int sign, int lane, int j)
 {
     const int e16 = 16 / esz;
@@ -204,24 +221,15 @@ size_t sptmm_pack_u16_bytes(int N, int S, int split_k)
 
 namespace sptmm {
 
-// One scheduling domain = the 32 lanes of a half-wavefront, which the LDS
-// serves in one pass when they hit 32 different banks (bank = row index mod 32
-// in every tile layout).  `owners` columns share the domain, each with `lanes`
-// lanes (owners*lanes == 32) and lanes*n entries.  Entries of a slot are chosen
-// bank by bank, fullest bank first, so that conflicts only appear once some
-// bank has run dry, and land in as few slots as possible.
-struct Domain {
-    int owners, lanes, n;
-    std::vector<std::vector<uint16_t>> entries;          // per owner
-    std::vector<std::vector<uint16_t>> cell;             // per owner: [slot][lane] -> index
-};
-
 void schedule(Domain &d)
 {
     const int no = d.owners, Lo = d.lanes, n = d.n;
     std::vector<std::array<std::vector<uint16_t>, 32>> pool(no);
-    for (int o = 0; o < no; ++o)
+    std::vector<int> wild(no);  // padding cells of each owner, free to take any bank
+    for (int o = 0; o < no; ++o) {
         for (uint16_t k : d.entries[o]) pool[o][k & 31].push_back(k);
+        wild[o] = n * Lo - (int)d.entries[o].size();
+    }
     d.cell.assign(no, std::vector<uint16_t>((size_t)n * Lo));
     std::vector<int> need(no);
     std::vector<std::vector<uint16_t>> pick(no);
@@ -245,9 +253,16 @@ void schedule(Domain &d)
                 int who = -1;
                 for (int o = 0; o < no; ++o)
                     if (need[o] > 0 && !pool[o][b].empty() && (who < 0 || pool[o][b].size() > pool[who][b].size())) who = o;
-                if (who < 0) continue;
-                pick[who].push_back(pool[who][b].back());
-                pool[who][b].pop_back();
+                if (who < 0) {  // no real entry left for this bank: a padding cell goes here
+                    for (int o = 0; o < no; ++o)
+                        if (need[o] > 0 && wild[o] > 0 && (who < 0 || wild[o] > wild[who])) who = o;
+                    if (who < 0) continue;
+                    pick[who].push_back((uint16_t)(d.zero_base + ((b - d.zero_base) & 31)));
+                    --wild[who];
+                } else {
+                    pick[who].push_back(pool[who][b].back());
+                    pool[who][b].pop_back();
+                }
                 --need[who];
                 --open;
             }
@@ -260,6 +275,7 @@ void schedule(Domain &d)
 }
 
 int u16_index_shift(int K) { return 4 * K <= 65535 ? 2 : 0; }
+int ragged_index_shift(int K) { return 4 * (K + 64) <= 65536 ? 2 : 0; }
 
 // Cells of the stream that belong to (column c, sign): calls f(task, lane, slot, i) for i = 0..half-1
 // in a fixed enumeration order: part-major, then half-wavefront, then slot, then lane.
@@ -450,184 +466,6 @@ int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int
 int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg)
 {
     return delta_walk(false, (void *)packed, pos, neg, K, N, S, split_k, bits);
-}
-
-// ------------------------------------------------------- striped gap streams
-// split_k 32 or 64 only.  Lane v of a column owns the rows of ONE residue class
-// mod 32 (rho = v % 32; with 64 lanes the class is cut in two ranges of j), i.e.
-// rows rho + 32*j, and stores the gaps of j in a byte.  All 32 lanes of a
-// half-wavefront therefore always sit on 32 different LDS banks, whatever the
-// data.  Lists of a task are padded to a common length n_t (a multiple of 4)
-// with entries that land on the zero rows K' = 32*ceil(K/32) + rho >= K of the
-// activation tile.  Task t lives at t*stride: 256 B of u16 first rows
-// [sign][lane], u32 n_t, u32 max_t n_t, 8 B zero, then the rounds of n_t gaps
-// per lane; stride = 272 + 128 * max_t n_t.
-}  // extern "C"
-
-namespace sptmm {
-
-struct StripedPlan {
-    Geometry g;
-    int J, Jh;                 // residue-class length ceil(K/32); first j of the upper half (64 lanes)
-    std::vector<int> n_task;   // padded entries per lane, per task
-    int n_min, n_max;
-    size_t stride, read_bytes; // task stride in the stream; bytes a GEMV actually reads
-    bool fits;                 // every gap (incl. the jump to the zero row) fits a byte
-};
-
-static inline int striped_lane(const StripedPlan &pl, int row)
-{
-    const int rho = row & 31, j = row >> 5;
-    return pl.g.L == 64 ? rho + 32 * (j >= pl.Jh) : rho;
-}
-
-// per-lane sorted sublists of one column and sign
-static void striped_split(const StripedPlan &pl, const uint16_t *lst, std::vector<std::vector<uint16_t>> &out)
-{
-    out.assign(pl.g.L, {});
-    for (int i = 0; i < pl.g.half; ++i) out[striped_lane(pl, lst[i])].push_back(lst[i]);
-}
-
-int striped_plan(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, StripedPlan *pl)
-{
-    if (int rc = check_shape(K, N, S)) return rc;
-    if (split_k != 32 && split_k != 64) return fail(SPTMM_ERR_INVALID, "striped gap streams need split_k 32 or 64");
-    if (int rc = make_geometry(N, S, split_k, 64, &pl->g)) return rc;
-    if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (K + 64 > 65535) return fail(SPTMM_ERR_UNSUPPORTED, "K too large for the striped gap stream");
-    const Geometry &g = pl->g;
-    pl->J = (K + 31) / 32;
-    pl->Jh = (pl->J + 1) / 2;
-    pl->n_task.assign(g.tasks, 4);
-    std::vector<int> bad(g.tasks, 0);
-    parallel_columns(g.tasks, [&](int t) {
-        std::vector<std::vector<uint16_t>> sub;
-        int most = 1;
-        for (int cc = 0; cc < g.G; ++cc)
-            for (int sign = 0; sign < 2; ++sign) {
-                const uint16_t *lst = (sign ? neg : pos) + (size_t)(t * g.G + cc) * g.half;
-                for (int i = 0; i < g.half; ++i)
-                    if (lst[i] >= K || (i && lst[i] <= lst[i - 1])) bad[t] = 1;
-                if (bad[t]) return;
-                striped_split(*pl, lst, sub);
-                for (auto &v : sub) {
-                    most = std::max(most, (int)v.size());
-                    for (size_t i = 1; i < v.size(); ++i)
-                        if ((v[i] - v[i - 1]) / 32 > 255) bad[t] = 2;
-                    const int last_j = v.empty() ? pl->J : v.back() >> 5;
-                    if (pl->J - last_j > 255) bad[t] = 2;
-                }
-            }
-        pl->n_task[t] = (most + 3) / 4 * 4;
-    });
-    pl->fits = true;
-    for (int t = 0; t < g.tasks; ++t) {
-        if (bad[t] == 1) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending and below K");
-        if (bad[t] == 2) pl->fits = false;
-    }
-    pl->n_max = *std::max_element(pl->n_task.begin(), pl->n_task.end());
-    pl->n_min = *std::min_element(pl->n_task.begin(), pl->n_task.end());
-    pl->stride = 272 + (size_t)128 * pl->n_max;
-    pl->read_bytes = 0;
-    for (int n : pl->n_task) pl->read_bytes += 272 + (size_t)128 * n;
-    return SPTMM_OK;
-}
-
-}  // namespace sptmm
-
-extern "C" {
-
-int sptmm_delta_striped_eligible(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k)
-{
-    StripedPlan pl;
-    if (split_k != 32 && split_k != 64) return 0;
-    if (K + 64 > 65535) return 0;
-    if (int rc = striped_plan(pos, neg, K, N, S, split_k, &pl)) return rc;
-    return pl.fits ? 1 : 0;
-}
-
-size_t sptmm_pack_delta_striped_bytes(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k,
-                                      size_t *read_bytes, int *n_min, int *n_max)
-{
-    StripedPlan pl;
-    if (striped_plan(pos, neg, K, N, S, split_k, &pl) || !pl.fits) return 0;
-    if (read_bytes) *read_bytes = pl.read_bytes;
-    if (n_min) *n_min = pl.n_min;
-    if (n_max) *n_max = pl.n_max;
-    return pl.stride * pl.g.tasks;
-}
-
-int sptmm_pack_delta_striped(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out)
-{
-    StripedPlan pl;
-    if (int rc = striped_plan(pos, neg, K, N, S, split_k, &pl)) return rc;
-    if (!pl.fits) return fail(SPTMM_ERR_UNSUPPORTED, "a gap does not fit a byte in the striped layout");
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const Geometry &g = pl.g;
-    uint8_t *base = (uint8_t *)out;
-    memset(base, 0, pl.stride * g.tasks);
-    parallel_columns(g.tasks, [&](int t) {
-        uint8_t *task = base + (size_t)t * pl.stride;
-        const int n = pl.n_task[t];
-        *(uint32_t *)(task + 256) = (uint32_t)n;
-        *(uint32_t *)(task + 260) = (uint32_t)pl.n_max;
-        std::vector<std::vector<uint16_t>> sub;
-        for (int cc = 0; cc < g.G; ++cc)
-            for (int sign = 0; sign < 2; ++sign) {
-                striped_split(pl, (sign ? neg : pos) + (size_t)(t * g.G + cc) * g.half, sub);
-                for (int v = 0; v < g.L; ++v) {
-                    const int lane = cc * g.L + v, zero_row = 32 * pl.J + (v & 31);
-                    const std::vector<uint16_t> &e = sub[v];
-                    *(uint16_t *)(task + sign * 128 + lane * 2) = (uint16_t)(e.empty() ? zero_row : e[0]);
-                    int prev = e.empty() ? zero_row : e[0];
-                    for (int i = 1; i < n; ++i) {
-                        const int row = i < (int)e.size() ? e[i] : zero_row;
-                        task[272 + slot_offset(n, 1, sign, lane, i)] = (uint8_t)((row - prev) / 32);
-                        prev = row;
-                    }
-                }
-            }
-    });
-    return SPTMM_OK;
-}
-
-int sptmm_unpack_delta_striped(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg)
-{
-    if (int rc = check_shape(K, N, S)) return rc;
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
-    if (split_k != 32 && split_k != 64) return fail(SPTMM_ERR_INVALID, "striped gap streams need split_k 32 or 64");
-    if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const uint8_t *base = (const uint8_t *)packed;
-    const uint32_t n_max = *(const uint32_t *)(base + 260);  // every task header repeats the largest n
-    if (n_max < 4 || n_max % 4 || n_max > 65536) return fail(SPTMM_ERR_INVALID, "not a striped gap stream");
-    const size_t stride = 272 + (size_t)128 * n_max;
-    std::vector<int> bad(g.tasks, 0);
-    parallel_columns(g.tasks, [&](int t) {
-        const uint8_t *task = base + (size_t)t * stride;
-        const int n = (int)*(const uint32_t *)(task + 256);
-        for (int cc = 0; cc < g.G; ++cc)
-            for (int sign = 0; sign < 2; ++sign) {
-                uint16_t *lst = (sign ? neg : pos) + (size_t)(t * g.G + cc) * g.half;
-                int cnt = 0;
-                for (int v = 0; v < g.L; ++v) {
-                    const int lane = cc * g.L + v;
-                    int row = *(const uint16_t *)(task + sign * 128 + lane * 2);
-                    for (int i = 0; i < n; ++i) {
-                        if (i) row += 32 * task[272 + slot_offset(n, 1, sign, lane, i)];
-                        if (row < K) {
-                            if (cnt < g.half) lst[cnt] = (uint16_t)row;
-                            ++cnt;
-                        }
-                    }
-                }
-                if (cnt != g.half) bad[t] = 1;
-                std::sort(lst, lst + std::min(cnt, g.half));
-            }
-    });
-    for (int t = 0; t < g.tasks; ++t)
-        if (bad[t]) return fail(SPTMM_ERR_INVALID, "striped gap stream does not hold S/2 rows per list");
-    return SPTMM_OK;
 }
 
 // ------------------------------------------------------------------------ i2s

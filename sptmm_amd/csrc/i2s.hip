@@ -191,12 +191,13 @@ int launch_copy(void *dst, const void *src, size_t bytes, void *stream)
 
 int launch_u16(const GemvArgs &a, ActType act, void *stream)
 {
+    if (a.ragged) return a.index_shift == 2 ? launch_ragged_u16_scaled(a, act, stream) : launch_ragged_u16_plain(a, act, stream);
     return a.index_shift == 2 ? launch_u16_scaled(a, act, stream) : launch_u16_plain(a, act, stream);
 }
 
 int launch_delta(const GemvArgs &a, ActType act, void *stream)
 {
-    if (a.delta_layout == 2) return launch_striped(a, act, stream);
+    if (a.ragged) return a.delta_bits == 8 ? launch_ragged_runs8(a, act, stream) : launch_ragged_runs16(a, act, stream);
     return a.delta_bits == 8 ? launch_runs8(a, act, stream) : launch_runs16(a, act, stream);
 }
 

@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstddef>
 #include <cstdint>
+#include <vector>
 
 #include "../../include/sptmm.h"
 
@@ -35,9 +36,31 @@ size_t slot_offset(int n_lane, int esz, int sign, int lane, int j);
 // u16 stream fields are row indices shifted left by this many bits (2 when 4*K fits 16 bits).
 int u16_index_shift(int K);
 
-// striped gap stream (formats.cpp): stride between tasks, smallest / largest per-task entry count
-struct StripedPlan;
-int striped_plan(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, StripedPlan *pl);
+// One scheduling domain of the u16 stream = the 32 lanes of a half-wavefront,
+// which the LDS serves in one pass when they hit 32 different banks (bank = row
+// index mod 32 in every tile layout).  `owners` columns share the domain, each
+// with `lanes` lanes (owners*lanes == 32) and lanes*n cells.  schedule() fills
+// cell[owner][slot*lanes + lane], choosing the entries of a slot bank by bank,
+// fullest bank first.  An owner with fewer than lanes*n entries gets the rest as
+// padding that may sit on any bank: zero rows zero_base + ((bank - zero_base) mod 32)
+// behind the activation tile.
+struct Domain {
+    int owners = 0, lanes = 0, n = 0;
+    int zero_base = 0;
+    std::vector<std::vector<uint16_t>> entries;  // per owner
+    std::vector<std::vector<uint16_t>> cell;     // per owner: [slot][lane] -> row
+};
+void schedule(Domain &d);
+
+// Geometry of a ragged stream (tasks carry their own entry count): as
+// make_geometry, with half = n_lane = 0.
+int make_ragged_geometry(int N, int split_k, int max_split, Geometry *g);
+// ragged u16 stream: fields are row << this (2 when 4*(K+64) fits 16 bits)
+int ragged_index_shift(int K);
+// ragged streams open with a 16-byte preamble {u32 magic, tasks, n_max, n_min} and one u16 entry
+// count per task; the tasks follow at the next multiple of 256 bytes
+constexpr uint32_t RAGGED_MAGIC = 0x52545053u;  // "SPTR"
+inline size_t ragged_counts_bytes(int tasks) { return ((size_t)16 + 2 * (size_t)tasks + 255) / 256 * 256; }
 
 // i2s tiling: 16 columns x 4 lanes per wave-load, 16 bytes (64 weights) per lane.
 inline int i2s_padded_k(int K) { return (K + 255) / 256 * 256; }
@@ -45,18 +68,18 @@ inline int i2s_padded_k(int K) { return (K + 255) / 256 * 256; }
 // ---- validation shared by packers and uploaders -----------------------------
 int check_shape(int K, int N, int S);
 
-// ---- device-side launchers (kernels.hip) --------------------------------------
+// ---- device-side launchers (i2s.hip and the lists_*.hip files) --------------------------------------
 struct GemvArgs {
     const void *w;      // device stream
     const void *X;      // device activations, row-major [M][K]
     void *C;            // device output, row-major [M][N]
     int M, K, N, half, split_k, n_lane, tasks, L, G, W;
     int delta_bits;
-    int delta_layout;   // 1 = contiguous runs, 2 = striped by row mod 32
-    int task_stride;    // striped: bytes between tasks
-    int n_min;          // striped: smallest per-task entry count
-    int n_max;          // striped: largest per-task entry count
     int index_shift;    // u16 stream: fields are row << index_shift
+    int ragged;         // the stream starts with a table of per-task entry counts; the next four fields apply
+    int task_stride;    // bytes between tasks
+    int counts_bytes;   // bytes of the count table, preamble included
+    int n_min, n_max;   // smallest / largest per-task entry count
     int compute_units;
     int lds_limit;
     // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each
@@ -72,7 +95,10 @@ int launch_u16_scaled(const GemvArgs &a, ActType act, void *stream);   // lists_
 int launch_u16_plain(const GemvArgs &a, ActType act, void *stream);    // lists_u16_plain.hip
 int launch_runs8(const GemvArgs &a, ActType act, void *stream);        // lists_runs8.hip
 int launch_runs16(const GemvArgs &a, ActType act, void *stream);       // lists_runs16.hip
-int launch_striped(const GemvArgs &a, ActType act, void *stream);      // lists_striped.hip
+int launch_ragged_u16_scaled(const GemvArgs &a, ActType act, void *stream);  // lists_ragged_u16_scaled.hip
+int launch_ragged_u16_plain(const GemvArgs &a, ActType act, void *stream);   // lists_ragged_u16_plain.hip
+int launch_ragged_runs8(const GemvArgs &a, ActType act, void *stream);       // lists_ragged_runs8.hip
+int launch_ragged_runs16(const GemvArgs &a, ActType act, void *stream);      // lists_ragged_runs16.hip
 int launch_delta(const GemvArgs &a, ActType act, void *stream);
 int launch_i2s(const GemvArgs &a, void *stream);
 int launch_copy(void *dst, const void *src, size_t bytes, void *stream);

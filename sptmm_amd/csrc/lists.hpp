@@ -1,5 +1,5 @@
 // Device code and launch templates shared by the list-stream translation units
-// (u16 lists, run gap streams, striped gap streams).  Each .hip file that
+// (u16 lists and run gap streams, balanced or ragged).  Each .hip file that
 // includes this header instantiates the kernels of one stream flavour, so the
 // flavours compile in parallel.
 #pragma once
@@ -56,25 +56,39 @@ __device__ __forceinline__ void gather(const unsigned char *lds, u32 addr, typen
     }
 }
 
-// MODE 0: fields are u16 row indices (already multiplied by 4 when PRE).
-// MODE 1 / 2: fields are 8- / 16-bit gaps in rows; MODE 3: 8-bit gaps in units
-// of 32 rows (striped stream).  `run` is the byte offset of the current row's
-// slot in the tile.  Consumes the low NBYTES of `d`.
+// Stream flavours (MODE):
+//   0  u16 row indices (already multiplied by 4 when PRE)
+//   1  8-bit gaps in rows, contiguous run per lane (256-byte task header: first row of every lane and sign)
+//   2  the same with 16-bit gaps
+// VAR (template flag of the kernels): ragged tasks.  The stream starts with a
+// table of per-task entry counts and the tasks sit at a fixed stride; lists
+// shorter than their task's count are padded with entries on the zero rows
+// behind the tile.
+template <int MODE> struct Flavour {
+    static constexpr bool GAP8 = MODE == 1;
+    static constexpr bool GAP16 = MODE == 2;
+    static constexpr int HDR = MODE == 0 ? 0 : 256;
+    static constexpr int ESZ = GAP8 ? 1 : 2;  // bytes per stream entry
+};
+constexpr int RAGGED_PREAMBLE = 16;  // {magic, tasks, n_max, n_min} in front of the u16 count table
+
+// `run` is the byte offset of the current row's slot in the tile.  Consumes the
+// low NBYTES of `d`.
 template <typename Act, int MT, int MODE, bool PRE, bool NEG, int NBYTES>
 __device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &run, typename Acc<Act>::type (&acc)[MT])
 {
     constexpr int SH = ilog2(slot_bytes<Act, MT>());
-    if constexpr (MODE == 1 || MODE == 3) {
+    if constexpr (Flavour<MODE>::GAP8) {
 #pragma unroll
         for (int b = 0; b < NBYTES; ++b) {
-            run += ((d >> (8 * b)) & 0xffu) << (MODE == 3 ? SH + 5 : SH);
+            run += ((d >> (8 * b)) & 0xffu) << SH;
             gather<Act, MT, NEG>(lds, run, acc);
         }
     } else {
 #pragma unroll
         for (int h = 0; h < NBYTES / 2; ++h) {
             u32 f = h ? (d >> 16) : (d & 0xffffu);
-            if constexpr (MODE == 2) {
+            if constexpr (Flavour<MODE>::GAP16) {
                 run += f << SH;
                 gather<Act, MT, NEG>(lds, run, acc);
             } else {
@@ -201,8 +215,9 @@ struct ListParams {
     const void *X;
     void *C;
     int M, K, N;
-    int n_lane, tasks, logL, W;  // n_lane: entries per lane per sign (striped stream: the smallest over all tasks)
-    int task_stride;             // striped stream: bytes between tasks
+    int n_lane, tasks, logL, W;  // n_lane: entries per lane per sign (ragged streams: the smallest over all tasks)
+    int task_stride;             // ragged streams: bytes between tasks
+    int counts_bytes;            // ragged streams: bytes of the count table (with its preamble) in front of the tasks
     int iters;  // tasks each wavefront walks: ceil(tasks / (gridDim.x * waves))
 };
 
@@ -232,18 +247,21 @@ __device__ __forceinline__ Round load_round(const uint4 *wp, int r)
     return x;
 }
 
-template <typename Act, int MT, int MODE, bool PRE>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR>
 struct ListsBody {
     typedef typename Acc<Act>::type A;
     typedef Stager<Act, MT> St;
     static constexpr int SLOT_OF = slot_bytes<Act, MT>();
-    static constexpr int ESZ = (MODE == 1 || MODE == 3) ? 1 : 2;   // bytes per stream entry
+    typedef Flavour<MODE> Fl;
+    static constexpr int ESZ = Fl::ESZ;               // bytes per stream entry
     static constexpr int E16 = 16 / ESZ;              // entries per 16-byte load
-    static constexpr int HDR = MODE == 3 ? 272 : (MODE ? 256 : 0);  // first rows (and entry count) of a gap-stream task
-    static constexpr int ZROWS = 64;                  // zero slots behind the tile (row K, and the striped stream's padding rows)
+    static constexpr int HDR = Fl::HDR;               // first rows of a gap-stream task
+    static constexpr bool GAPS = Fl::GAP8 || Fl::GAP16;
+    static constexpr int ZROWS = 64;                  // zero slots behind the tile (row K, and the padding rows)
     static constexpr int SH = ilog2(SLOT_OF);
     static constexpr int SLOT = SLOT_OF;
     static constexpr int RING = 8;                    // rounds in flight on the generic path
+    static constexpr int XMAX = VAR ? 2 : 0;          // ragged tasks on the straight-line path: full rounds beyond RF a task may have
 #ifndef SPTMM_EARLY
 #define SPTMM_EARLY 2
 #endif
@@ -258,13 +276,13 @@ struct ListsBody {
         // value of every round alive to sum them in one tree at the end.
 #pragma unroll
         for (int m = 0; m < MT; ++m) asm volatile("" : "+v"(acc[m]));
-        if constexpr (MODE != 0) asm volatile("" : "+v"(runp), "+v"(runq));
+        if constexpr (GAPS) asm volatile("" : "+v"(runp), "+v"(runq));
     }
 
-    // RF > 0: the task has exactly RF full rounds and all of them live in
-    // registers, loaded and consumed in straight-line code (so every wait on the
-    // stream is for one round only).  RF == 0: any number of rounds, through a
-    // ring of RING rounds in flight.
+    // RF > 0: the task has exactly RF full rounds (ragged: RF to RF + XMAX) and
+    // all of them live in registers, loaded and consumed in straight-line code
+    // (so every wait on the stream is for one round only).  RF == 0: any number
+    // of rounds, through a ring of RING rounds in flight.
     template <int RF>
     static __device__ __forceinline__ void run(const ListParams &p, unsigned char *smem)
     {
@@ -273,8 +291,10 @@ struct ListsBody {
         const int tid = threadIdx.x, nt = blockDim.x;
         const int lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
         const int m0 = blockIdx.y * MT;
-        const size_t task_bytes = MODE == 3 ? (size_t)p.task_stride : HDR + (size_t)128 * ESZ * p.n_lane;
-        // striped stream: tasks differ in length; p.n_lane is the shortest, which is all the prologue may assume
+        const size_t task_bytes = VAR ? (size_t)p.task_stride : HDR + (size_t)128 * ESZ * p.n_lane;
+        const uint8_t *const tasks_base = p.w + (VAR ? p.counts_bytes : 0);
+        const unsigned short *const counts = reinterpret_cast<const unsigned short *>(p.w + RAGGED_PREAMBLE);
+        // ragged: tasks differ in length; p.n_lane is the shortest, which is all the prologue may assume
         const int R0 = p.n_lane / E16;
         int task = blockIdx.x * waves + wave;
         const int task_step = gridDim.x * waves;
@@ -289,14 +309,15 @@ struct ListsBody {
             const int item = tid + i * nt;
             St::load(X, p.M, p.K, m0, item < items ? item : items - 1, xr[i]);
         }
-#ifdef SPTMM_XBARRIER
-        __builtin_amdgcn_s_barrier();
-#endif
+        // ragged: the first task's entry count travels with the activation loads, so it is there
+        // long before the tile is; every later count is asked for one task ahead
+        int n_ahead = p.n_lane;
+        if constexpr (VAR) n_ahead = counts[task < p.tasks ? task : 0];
 
         // 2. ... then the first rounds of the first task's stream ...
         Round buf[NB];
         {
-            const uint4 *wp = reinterpret_cast<const uint4 *>(p.w + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
+            const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
             if constexpr (RF > 0) {
 #pragma unroll
                 for (int i = 0; i < (RF < EARLY ? RF : EARLY); ++i) buf[i] = load_round(wp, i);
@@ -311,12 +332,12 @@ struct ListsBody {
         for (int i = 0; i < St::XI; ++i)
             if (tid + i * nt < items) St::store(smem, tid + i * nt, xr[i]);
         if constexpr (RF > EARLY) {
-            const uint4 *wp = reinterpret_cast<const uint4 *>(p.w + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
+            const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
 #pragma unroll
             for (int i = EARLY; i < RF; ++i) buf[i] = load_round(wp, i);
         } else if constexpr (RF == 0) {
             if (R0 > 0) {
-                const uint4 *wp = reinterpret_cast<const uint4 *>(p.w + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
+                const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
 #pragma unroll
                 for (int i = EARLY; i < RING; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
             }
@@ -333,16 +354,20 @@ struct ListsBody {
         const int L = 1 << p.logL;
         for (int it = 0; it < p.iters; ++it, task += task_step) {
             const bool active = task < p.tasks;
-            const uint8_t *tb = p.w + (size_t)(active ? task : 0) * task_bytes;
+            const uint8_t *tb = tasks_base + (size_t)(active ? task : 0) * task_bytes;
             const uint4 *wp = reinterpret_cast<const uint4 *>(tb + HDR) + lane;
             u32 runp = 0, runq = 0;
             int n_lane = p.n_lane;
-            if constexpr (MODE != 0) {
+            if constexpr (GAPS) {
                 const unsigned short *rs = reinterpret_cast<const unsigned short *>(tb);
                 runp = (u32)rs[lane] << SH;
                 runq = (u32)rs[64 + lane] << SH;
             }
-            if constexpr (MODE == 3 && RF == 0) n_lane = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int *>(tb + 256));
+            if constexpr (VAR) {
+                n_lane = __builtin_amdgcn_readfirstlane(n_ahead);
+                const int nxt = task + task_step;
+                n_ahead = counts[nxt < p.tasks ? nxt : 0];
+            }
             const int R = n_lane / E16, rem = n_lane - R * E16;
             A acc[MT];
 #pragma unroll
@@ -360,11 +385,17 @@ struct ListsBody {
 #pragma unroll
                         for (int i = 0; i < RING; ++i) buf[i] = load_round(wp, i < R ? i : R - 1);
                     }
-                } else if (MODE == 3) {  // this task may be longer than the shortest one the prologue assumed
+                } else if (VAR) {  // this task may be longer than the shortest one the prologue assumed
 #pragma unroll
                     for (int i = 0; i < RING; ++i)
                         if (i >= R0 && i < R) buf[i] = load_round(wp, i);
                 }
+            }
+            Round xb[XMAX > 0 ? XMAX : 1];
+            if constexpr (RF > 0 && XMAX > 0) {
+#pragma unroll
+                for (int x = 0; x < XMAX; ++x)
+                    if (RF + x < R) xb[x] = load_round(wp, RF + x);
             }
             // ragged tail, requested now and eaten last: at most one round each of 8, 4, 2 (and 1) bytes per lane
             uint2 t8p = make_uint2(0, 0), t8q = make_uint2(0, 0);
@@ -418,6 +449,11 @@ struct ListsBody {
             } else {
 #pragma unroll
                 for (int i = 0; i < RF; ++i) eat(smem, buf[i], runp, runq, acc);
+                if constexpr (XMAX > 0) {
+#pragma unroll
+                    for (int x = 0; x < XMAX; ++x)
+                        if (RF + x < R) eat(smem, xb[x], runp, runq, acc);
+                }
             }
             if (rem) {
                 if (rem & (8 / ESZ)) {
@@ -480,11 +516,11 @@ struct ListsBody {
 // wavefronts then walk tasks blockIdx.x*waves + wave, + gridDim.x*waves, ...
 // blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
 // exactly RF full rounds (straight-line body); RF == 0: any length (ring).
-template <typename Act, int MT, int MODE, bool PRE, int RF>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
 __global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    ListsBody<Act, MT, MODE, PRE>::template run<RF>(p, smem);
+    ListsBody<Act, MT, MODE, PRE, VAR>::template run<RF>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -496,14 +532,14 @@ struct BatchPtrs {
     void *C[BATCH_MAX];
 };
 
-template <typename Act, int MT, int MODE, bool PRE, int RF>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
 __global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel_batched(ListParams p, BatchPtrs b)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     p.w = b.w[blockIdx.z];
     p.X = b.X[blockIdx.z];
     p.C = b.C[blockIdx.z];
-    ListsBody<Act, MT, MODE, PRE>::template run<RF>(p, smem);
+    ListsBody<Act, MT, MODE, PRE, VAR>::template run<RF>(p, smem);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -522,7 +558,7 @@ static inline int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &g
     return SPTMM_OK;
 }
 
-template <typename Act, int MT, int MODE, bool PRE, int RF>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
 static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
 {
     // Wavefronts per workgroup: fill the CUs with one workgroup each, and when a
@@ -530,8 +566,16 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // fewest wavefront slots over the task loop.
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
     static const int tune_wpb = getenv("SPTMM_WAVES_PER_WG") ? atoi(getenv("SPTMM_WAVES_PER_WG")) : 0;
-    static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 1;
-    const int slots = cus * (tune_wgs > 0 ? tune_wgs : 1);  // workgroups resident at once
+    static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
+    constexpr int SLOT = slot_bytes<Act, MT>();
+    const size_t tile = (size_t)(a.K + 64) * SLOT + (size_t)LISTS_MAX_WAVES * MT * sizeof(typename Acc<Act>::type);
+    // Workgroups resident per CU.  A wavefront asks for its next task's stream only when it is
+    // done with the current one, so once a CU's share exceeds one workgroup of single-task
+    // wavefronts, a second resident workgroup fills those gaps (measured on MI355X, K=2560
+    // N=13824 split_k=32: 11.4 -> 6.3 us); a third does not fit the register file.
+    int wgs = tune_wgs > 0 ? tune_wgs : (!a.batch && a.tasks > LISTS_MAX_WAVES * cus ? 2 : 1);
+    while (wgs > 1 && tile * wgs > (size_t)a.lds_limit) --wgs;
+    const int slots = cus * wgs;  // workgroups resident at once
     int wpb = a.W, best = 1 << 30;
     for (int w = a.W; w <= LISTS_MAX_WAVES; w += a.W) {
         int blocks = (a.tasks + w - 1) / w;
@@ -547,15 +591,14 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     const int blocks = (a.tasks + wpb - 1) / wpb;
     const int grid_x = blocks < slots ? blocks : slots;
     const int iters = (blocks + grid_x - 1) / grid_x;
-    ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, MODE == 3 ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
-                 a.task_stride, iters};
-    constexpr int SLOT = slot_bytes<Act, MT>();
+    ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
+                 a.task_stride, a.counts_bytes, iters};
     size_t lds = (size_t)(a.K + 64) * SLOT + (size_t)wpb * MT * sizeof(typename Acc<Act>::type);
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     if (a.batch) {
         if constexpr (sizeof(Act) == 1) {
-            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, RF>;
+            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, VAR, RF>;
             static std::atomic<size_t> lds_granted_b{48 * 1024};
             if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_b)) return rc;
             for (int first = 0; first < a.batch; first += BATCH_MAX) {
@@ -576,7 +619,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take int8 activations");
         }
     }
-    auto kern = lists_kernel<Act, MT, MODE, PRE, RF>;
+    auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF>;
     static std::atomic<size_t> lds_granted{48 * 1024};
     if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
     hipLaunchKernelGGL(kern, grid, block, lds, st, p);
@@ -585,42 +628,49 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
 }
 
 // Straight-line bodies exist for the int8 paths of the u16 and 8-bit run streams
-// with 1, 2, 3, 4, 6 or 8 full rounds per task; everything else takes the ring.
-template <typename Act, int MT, int MODE, bool PRE>
+// with 1, 2, 3, 4, 6 or 8 full rounds per task (ragged streams: for the shortest
+// task, when the longest has at most XMAX more); everything else takes the ring.
+template <typename Act, int MT, int MODE, bool PRE, bool VAR>
 static int launch_lists_t(const GemvArgs &a, hipStream_t st)
 {
     if constexpr (sizeof(Act) == 1 && MODE < 2) {
-        switch (a.n_lane / (MODE == 1 ? 16 : 8)) {
-        case 1: return launch_lists_rf<Act, MT, MODE, PRE, 1>(a, st);
-        case 2: return launch_lists_rf<Act, MT, MODE, PRE, 2>(a, st);
-        case 3: return launch_lists_rf<Act, MT, MODE, PRE, 3>(a, st);
-        case 4: return launch_lists_rf<Act, MT, MODE, PRE, 4>(a, st);
-        case 6: return launch_lists_rf<Act, MT, MODE, PRE, 6>(a, st);
-        case 8: return launch_lists_rf<Act, MT, MODE, PRE, 8>(a, st);
+        constexpr int E16 = MODE == 1 ? 16 : 8;
+        int rf = (VAR ? a.n_min : a.n_lane) / E16;
+        if constexpr (VAR) {
+            rf = rf >= 8 ? 8 : rf >= 6 ? 6 : rf == 5 ? 4 : rf;
+            if (a.n_max / E16 - rf > ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) rf = 0;
+        }
+        switch (rf) {
+        case 1: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 1>(a, st);
+        case 2: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 2>(a, st);
+        case 3: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 3>(a, st);
+        case 4: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 4>(a, st);
+        case 6: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 6>(a, st);
+        case 8: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 8>(a, st);
         default: break;
         }
     }
-    return launch_lists_rf<Act, MT, MODE, PRE, 0>(a, st);
+    return launch_lists_rf<Act, MT, MODE, PRE, VAR, 0>(a, st);
 }
 
-template <typename Act, int MODE, bool PRE>
+template <typename Act, int MODE, bool PRE, bool VAR>
 static int launch_lists_m(const GemvArgs &a, hipStream_t st)
 {
     const size_t lim = (size_t)a.lds_limit - 256;
     if constexpr (sizeof(Act) == 1) {
-        if (a.M >= 5 && (size_t)(a.K + 64) * slot_bytes<Act, 8>() <= lim) return launch_lists_t<Act, 8, MODE, PRE>(a, st);
+        if (a.M >= 5 && (size_t)(a.K + 64) * slot_bytes<Act, 8>() <= lim) return launch_lists_t<Act, 8, MODE, PRE, VAR>(a, st);
     }
-    if (a.M >= 2 && (size_t)(a.K + 64) * slot_bytes<Act, 4>() <= lim) return launch_lists_t<Act, 4, MODE, PRE>(a, st);
-    return launch_lists_t<Act, 1, MODE, PRE>(a, st);
+    if (a.M >= 2 && (size_t)(a.K + 64) * slot_bytes<Act, 4>() <= lim) return launch_lists_t<Act, 4, MODE, PRE, VAR>(a, st);
+    return launch_lists_t<Act, 1, MODE, PRE, VAR>(a, st);
 }
 
-template <int MODE, bool PRE>
+template <int MODE, bool PRE, bool VAR>
 static int launch_lists_a(const GemvArgs &a, ActType act, hipStream_t st)
 {
     switch (act) {
-    case ACT_I8: return launch_lists_m<int8_t, MODE, PRE>(a, st);
-    case ACT_F16: return launch_lists_m<_Float16, MODE, PRE>(a, st);
-    case ACT_F32: return launch_lists_m<float, MODE, PRE>(a, st);
+    case ACT_I8: return launch_lists_m<int8_t, MODE, PRE, VAR>(a, st);
+    case ACT_F16: return launch_lists_m<_Float16, MODE, PRE, VAR>(a, st);
+    case ACT_F32: return launch_lists_m<float, MODE, PRE, VAR>(a, st);
     }
     return fail(SPTMM_ERR_INVALID, "unknown activation type");
 }

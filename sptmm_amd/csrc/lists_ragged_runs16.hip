@@ -1,0 +1,8 @@
+// ragged run gap stream (per-task entry counts), 16-bit gaps.
+#include "lists.hpp"
+
+namespace sptmm {
+
+int launch_ragged_runs16(const GemvArgs &a, ActType act, void *stream) { return launch_lists_a<2, false, true>(a, act, (hipStream_t)stream); }
+
+}  // namespace sptmm

@@ -1,8 +1,8 @@
-// gap stream, contiguous runs, 16-bit gaps.
+// run gap stream, 16-bit gaps.
 #include "lists.hpp"
 
 namespace sptmm {
 
-int launch_runs16(const GemvArgs &a, ActType act, void *stream) { return launch_lists_a<2, false>(a, act, (hipStream_t)stream); }
+int launch_runs16(const GemvArgs &a, ActType act, void *stream) { return launch_lists_a<2, false, false>(a, act, (hipStream_t)stream); }
 
 }  // namespace sptmm

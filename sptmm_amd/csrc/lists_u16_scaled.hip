@@ -3,6 +3,6 @@
 
 namespace sptmm {
 
-int launch_u16_scaled(const GemvArgs &a, ActType act, void *stream) { return launch_lists_a<0, true>(a, act, (hipStream_t)stream); }
+int launch_u16_scaled(const GemvArgs &a, ActType act, void *stream) { return launch_lists_a<0, true, false>(a, act, (hipStream_t)stream); }
 
 }  // namespace sptmm

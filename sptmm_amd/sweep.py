@@ -3,6 +3,10 @@
     python -m sptmm_amd.sweep layer     # BitNet-b1.58-2B decoder layer: q/o, k/v, gate/up (K=2560), down (K=6912)
     python -m sptmm_amd.sweep large     # K=13824 N=5120 S=8320, M in {1, 8, 16}
     python -m sptmm_amd.sweep headline  # K=6912 N=2560 S=4096, M in {1, 4}
+    python -m sptmm_amd.sweep fused     # the layer with q+k+v (N=3840) and gate+up (N=13824) as single launches,
+                                        # the fusions the reference benchmarks (main.cu:1107-1190): 4 launches per layer
+    python -m sptmm_amd.sweep ragged    # the same four launches on matrices with independent entries (30 % +1, 30 % -1):
+                                        # columns differ in nonzeros, streams carry per-task counts
 
 Per shape and encoding: microseconds per GEMV launched alone (cache-warm = the same stream every launch;
 HBM-cold = rotating over enough device copies to exceed the 256 MB last-level cache) and, for the list
@@ -20,6 +24,8 @@ from . import _capi as sp
 
 PEAK_GBPS = 8000.0
 LAYER = [("q/o", 2560, 2560, 1536, 2), ("k/v", 2560, 640, 1536, 2), ("gate/up", 2560, 6912, 1536, 2),
+         ("down", 6912, 2560, 4160, 1)]
+FUSED = [("qkv", 2560, 3840, 1536, 1), ("o", 2560, 2560, 1536, 1), ("gate+up", 2560, 13824, 1536, 1),
          ("down", 6912, 2560, 4160, 1)]
 
 
@@ -48,14 +54,21 @@ def time_weights(w, X, M, N, st, batched: bool):
     return warm, cold, bat
 
 
-def run_shape(name, K, N, S, Ms, splits, st, rows):
-    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+def run_shape(name, K, N, S, Ms, splits, st, rows, iid=None):
+    if iid is None:
+        W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    else:
+        W = sp.generate_ternary_iid(K, N, 0x5EED ^ N, *iid)
     for M in Ms:
         X = sp.make_x_i8(0xC0FFEE ^ M, M, K)
         ref = None
-        cands = [("u16/%d" % s, lambda s=s: sp.Weights.upload_u16(pos, neg, K, s)) for s in splits if (S // 2) % s == 0]
-        cands += [("delta/%d" % s, lambda s=s: sp.Weights.upload_delta(pos, neg, K, s)) for s in splits
-                  if s <= 64 and (S // 2) % s == 0]
+        if iid is None:
+            cands = [("u16/%d" % s, lambda s=s: sp.Weights.upload_u16(pos, neg, K, s)) for s in splits if (S // 2) % s == 0]
+            cands += [("delta/%d" % s, lambda s=s: sp.Weights.upload_delta(pos, neg, K, s)) for s in splits
+                      if s <= 64 and (S // 2) % s == 0]
+        else:
+            cands = [("u16/%d" % s, lambda s=s: sp.Weights.upload_dense(W, sp.KIND_U16, s)) for s in splits]
+            cands += [("delta/%d" % s, lambda s=s: sp.Weights.upload_dense(W, sp.KIND_DELTA, s)) for s in splits if s <= 64]
         cands += [("i2s", lambda: sp.Weights.upload_i2s(W))]
         for enc, mk in cands:
             w = mk()
@@ -63,7 +76,7 @@ def run_shape(name, K, N, S, Ms, splits, st, rows):
             if ref is None:
                 ref = got
             ok = bool((got == ref).all())
-            nbytes = w.nbytes + M * K + 4 * M * N
+            nbytes = w.info["stream_bytes"] + M * K + 4 * M * N  # what one GEMV reads and writes
             warm, cold, bat = time_weights(w, X, M, N, st, enc != "i2s")
             w.free()
             rows.append({"shape": name, "K": K, "N": N, "S": S, "M": M, "enc": enc, "bytes": nbytes, "ok": ok,
@@ -82,24 +95,27 @@ def main(argv):
     info = sp.device_init(0)
     st = sp.Stream()
     rows = []
-    if which == "layer":
-        for name, K, N, S, _ in LAYER:
-            run_shape(name, K, N, S, (1, 4), (8, 16, 32, 64), st, rows)
+    if which in ("layer", "fused", "ragged"):
+        shapes = LAYER if which == "layer" else FUSED
+        for name, K, N, S, _ in shapes:
+            run_shape(name, K, N, S, (1, 4), (8, 16, 32, 64) if which == "layer" else (16, 32, 64), st, rows,
+                      iid=(0.3, 0.3) if which == "ragged" else None)
         for M in (1, 4):
             for kind in ("u16", "delta", "i2s"):
                 tot_w = tot_c = 0.0
-                for name, K, N, S, mult in LAYER:
+                for name, K, N, S, mult in shapes:
                     best = [r for r in rows if r["shape"] == name and r["M"] == M and r["enc"].startswith(kind)]
                     tot_w += mult * min(r["warm_us"] for r in best)
                     tot_c += mult * min(r["cold_us"] for r in best)
-                print("layer sum (7 GEMVs, best split per shape) M=%d %-5s: warm %.1f us  cold %.1f us" % (M, kind, tot_w, tot_c))
+                print("layer sum (%d launches, best split per shape) M=%d %-5s: warm %.1f us  cold %.1f us"
+                      % (sum(m for *_, m in shapes), M, kind, tot_w, tot_c))
                 rows.append({"shape": "layer_sum", "M": M, "enc": kind, "warm_us": round(tot_w, 2), "cold_us": round(tot_c, 2)})
     elif which == "large":
         run_shape("large", 13824, 5120, 8320, (1, 8, 16), (32, 64), st, rows)
     elif which == "headline":
         run_shape("headline", 6912, 2560, 4096, (1, 4), (16, 32, 64), st, rows)
     else:
-        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline")
+        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged")
     assert all(r.get("ok", True) for r in rows), "encodings disagree"
     print(json.dumps({"device": info["arch"], "rows": rows}))
 

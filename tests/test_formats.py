@@ -208,38 +208,3 @@ def test_i2s_rejects_non_ternary():
     W[3, 5] = 2
     with pytest.raises(sp.SptmmError):
         sp.pack_i2s(W)
-
-
-@pytest.mark.parametrize("split", [32, 64])
-@pytest.mark.parametrize("K,N,S", [(2560, 64, 1536), (6912, 32, 4096), (6912, 16, 4160), (512, 32, 256), (6912, 16, 64)])
-def test_striped_delta_round_trip_and_bank_rule(K, N, S, split):
-    _, pos, neg = sp.generate_ternary(K, N, S)
-    if (S // 2) % split:
-        return
-    assert sp.delta_striped_eligible(pos, neg, K, split)
-    pk, meta = sp.pack_delta_striped(pos, neg, K, split)
-    p2, n2 = sp.unpack_delta_striped(pk, K, N, S, split)
-    assert (p2 == pos).all() and (n2 == neg).all()
-    tasks = N // (64 // split)
-    stride = 272 + 128 * meta["n_max"]
-    assert pk.nbytes == tasks * stride
-    ns = [int(pk[t * stride + 256: t * stride + 260].view(np.uint32)[0]) for t in range(tasks)]
-    assert min(ns) == meta["n_min"] and max(ns) == meta["n_max"] and all(n % 4 == 0 for n in ns)
-    assert meta["read_bytes"] == sum(272 + 128 * n for n in ns)
-    # every lane starts on its own residue class: lane % 32 == first row % 32 (both signs), and gaps keep it there
-    for t in (0, tasks - 1):
-        first = pk[t * stride: t * stride + 256].view(np.uint16).reshape(2, 64)
-        assert ((first % 32) == (np.arange(64) % 32)).all()
-    # padding cost at the headline density (lists of ~64 rows per lane)
-    if S >= 4096 and split == 32:
-        assert meta["read_bytes"] <= 1.45 * S * N
-
-
-def test_striped_delta_not_eligible_for_large_k_or_other_splits():
-    K, N, S = 16384, 16, 512          # 512 residue steps per class: the jump to the zero row exceeds a byte
-    _, pos, neg = sp.generate_ternary(K, N, S)
-    assert not sp.delta_striped_eligible(pos, neg, K, 32)
-    _, pos, neg = sp.generate_ternary(2560, 16, 1536)
-    assert not sp.delta_striped_eligible(pos, neg, 2560, 16)
-    with pytest.raises(sp.SptmmError):
-        sp.pack_delta_striped(pos, neg, 2560, 16)

@@ -153,27 +153,25 @@ def test_delta_headline_shape_int8_bit_exact(split):
     say("delta i8 split", split)
     _, pos, neg = matrix(K, N, S)
     w = sp.Weights.upload_delta(pos, neg, K, split)
-    assert w.info["delta_bits"] == 8 and w.info["delta_layout"] == 1
+    assert w.info["delta_bits"] == 8 and w.info["ragged"] == 0
     for M in (1, 4):
         X = x_i8(0xC0FFEE ^ M, M, K)
         assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), M
     w.free()
 
 
-@pytest.mark.parametrize("layout", [1, 2])
 @pytest.mark.parametrize("K,N,S,split", [(6912, 2560, 4096, 32), (6912, 2560, 4096, 64), (2560, 640, 1536, 32),
                                          (6912, 64, 4160, 32), (512, 48, 256, 64), (6912, 32, 64, 32)])
-def test_delta_both_layouts_bit_exact(K, N, S, split, layout):
+def test_delta_all_activation_types(K, N, S, split):
     _, pos, neg = matrix(K, N, S)
-    w = sp.Weights.upload_delta(pos, neg, K, split, layout=layout)
-    assert w.info["delta_layout"] == layout
+    w = sp.Weights.upload_delta(pos, neg, K, split)
     for M in (1, 3, 4, 8):
-        say("delta layout", layout, K, N, S, "split", split, "M", M, "bits", w.info["delta_bits"])
-        X = x_i8(31 * M + layout, M, K)
+        say("delta", K, N, S, "split", split, "M", M, "bits", w.info["delta_bits"])
+        X = x_i8(31 * M + 1, M, K)
         assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), M
-    Xh = oracle.make_x_normal(layout, 2, K, np.float16)
+    Xh = oracle.make_x_normal(1, 2, K, np.float16)
     check_fp(w.matmul(Xh), oracle.sptmm_f64(Xh, pos, neg), S)
-    Xf = oracle.make_x_normal(layout, 1, K, np.float32)
+    Xf = oracle.make_x_normal(1, 1, K, np.float32)
     check_fp(w.matmul(Xf), oracle.sptmm_f64(Xf, pos, neg), S)
     w.free()
 
@@ -220,7 +218,7 @@ def test_delta_fp16_config2():
 def test_delta_ragged_sparse_and_16bit(K, N, S, splits):
     _, pos, neg = matrix(K, N, S)
     for split in splits:
-        w = sp.Weights.upload_delta(pos, neg, K, split, layout=1)
+        w = sp.Weights.upload_delta(pos, neg, K, split)
         bits = w.info["delta_bits"]
         assert bits == sp.delta_bits(pos, neg, split)
         for M in (1, 4, 5):
