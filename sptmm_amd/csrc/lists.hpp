@@ -5,6 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 
@@ -561,33 +562,53 @@ static inline int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &g
 template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
 static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
 {
-    // Wavefronts per workgroup: fill the CUs with one workgroup each, and when a
-    // CU gets more than LISTS_MAX_WAVES tasks pick the count that wastes the
-    // fewest wavefront slots over the task loop.
+    // Launch shape: g workgroups resident per CU, w wavefronts each.  A wavefront asks for its
+    // next task's stream only when it is done with the current one, so what hides the memory
+    // latency is the number of tasks in flight per CU, R = g*w.  The loop over tasks costs
+    // iterations * max(R, R_lat) in units of one task's streaming time at the CU's share of the
+    // HBM bandwidth (R_lat = tasks needed in flight to cover ~2 us of latency at 8 TB/s over the
+    // CUs, i.e. ~62 KB per CU); R is bounded by the kernel's register footprint and the LDS the
+    // tiles take.  Measured on MI355X, K=2560 N=13824 split_k=32: one workgroup per CU 11.4 us,
+    // two 6.3 us; the headline shape has 5 tasks per CU and stays at one workgroup of 5.
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
     static const int tune_wpb = getenv("SPTMM_WAVES_PER_WG") ? atoi(getenv("SPTMM_WAVES_PER_WG")) : 0;
     static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
     constexpr int SLOT = slot_bytes<Act, MT>();
-    const size_t tile = (size_t)(a.K + 64) * SLOT + (size_t)LISTS_MAX_WAVES * MT * sizeof(typename Acc<Act>::type);
-    // Workgroups resident per CU.  A wavefront asks for its next task's stream only when it is
-    // done with the current one, so once a CU's share exceeds one workgroup of single-task
-    // wavefronts, a second resident workgroup fills those gaps (measured on MI355X, K=2560
-    // N=13824 split_k=32: 11.4 -> 6.3 us); a third does not fit the register file.
-    int wgs = tune_wgs > 0 ? tune_wgs : (!a.batch && a.tasks > LISTS_MAX_WAVES * cus ? 2 : 1);
-    while (wgs > 1 && tile * wgs > (size_t)a.lds_limit) --wgs;
-    const int slots = cus * wgs;  // workgroups resident at once
-    int wpb = a.W, best = 1 << 30;
-    for (int w = a.W; w <= LISTS_MAX_WAVES; w += a.W) {
-        int blocks = (a.tasks + w - 1) / w;
-        int grid = blocks < slots ? blocks : slots;
-        int iters = (blocks + grid - 1) / grid;
-        int cost = iters * w;
-        if (cost < best || (cost == best && w > wpb)) {
-            best = cost;
-            wpb = w;
+    const size_t tile = (size_t)(a.K + 64) * SLOT;
+    static std::atomic<int> vgprs{0};  // of the single-GEMV kernel of this instantiation
+    int regs = vgprs.load(std::memory_order_relaxed);
+    if (!regs) {
+        hipFuncAttributes fa;
+        hipError_t e = hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(lists_kernel<Act, MT, MODE, PRE, VAR, RF>));
+        if (e != hipSuccess) return hip_fail(e, "hipFuncGetAttributes");
+        regs = fa.numRegs > 0 ? fa.numRegs : 128;
+        vgprs.store(regs, std::memory_order_relaxed);
+    }
+    const int waves_per_simd = std::max(1, std::min(8, 512 / ((regs + 7) / 8 * 8)));
+    const double task_kb = (VAR ? a.task_stride : Flavour<MODE>::HDR + 128 * Flavour<MODE>::ESZ * a.n_lane) / 1024.0;
+    const double r_lat = 62.0 / (task_kb > 0.25 ? task_kb : 0.25);
+    int wpb = a.W, wgs = 1;
+    double best = 1e30;
+    for (int g = 1; g <= (a.batch ? 1 : 3); ++g) {
+        if (tune_wgs > 0 && g != tune_wgs) continue;
+        for (int w = a.W; w <= LISTS_MAX_WAVES; w += a.W) {
+            if (g > 1 && g * w > 4 * waves_per_simd) continue;  // the register file of the CU's 4 SIMDs
+            if (g > 1 && g * (tile + (size_t)w * MT * 4) > (size_t)a.lds_limit) continue;
+            const int blocks = (a.tasks + w - 1) / w;
+            const int grid = blocks < cus * g ? blocks : cus * g;
+            const int iters = (blocks + grid - 1) / grid;
+            const double r = (double)g * w;
+            // + each workgroup stages the tile once; a bubble per extra pass; when latency-bound, spread over more CUs
+            const double cost = iters * (r > r_lat ? r : r_lat) + 0.05 * g + 0.25 * (iters - 1) + 0.001 * r;
+            if (cost < best - 1e-9) {
+                best = cost;
+                wpb = w;
+                wgs = g;
+            }
         }
     }
     if (tune_wpb > 0 && tune_wpb <= LISTS_MAX_WAVES && tune_wpb % a.W == 0) wpb = tune_wpb;
+    const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
     const int grid_x = blocks < slots ? blocks : slots;
     const int iters = (blocks + grid_x - 1) / grid_x;
