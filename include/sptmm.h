@@ -91,9 +91,12 @@ int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S
 int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg);
 
 /* Gap streams; replaces W_map_delta2_d / W_map_delta2_div256 of main.cu:376-413.
- * Each lane owns a contiguous run of the sorted list: a 16-bit restart index
- * followed by its gaps.  sptmm_delta_bits() returns 8 when every in-run gap
- * fits a byte, else 16 (the reference narrows silently, main.cu:380-383).
+ * Each lane owns a contiguous run of the sorted list: a 16-bit first row
+ * followed by its gaps.  16-bit gaps are unsigned and ascending.  8-bit gaps are
+ * SIGNED: a lane visits its run in an order chosen by the packer (steps within
+ * -128..127) so that the 32 lanes of a half-wavefront gather from different LDS
+ * banks.  sptmm_delta_bits() returns 8 when every in-run gap of the sorted lists
+ * is at most 127, else 16 (the reference narrows silently, main.cu:380-383).
  * split_k in {8,16,32,64}. */
 int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int split_k);
 size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits);

@@ -274,6 +274,123 @@ void schedule(Domain &d)
     }
 }
 
+bool schedule_runs(RunDomain &d, int window)
+{
+    const int n = d.n;
+    struct Lane {
+        std::vector<char> seen;   // visited entries
+        int lo = 0, cur = -1;     // oldest entry not visited yet; row visited last
+        std::vector<int> cand;    // this step's candidates (entry indices), most urgent bank first
+        int pick = -1;
+    } lane[32];
+    int demand[32] = {0};         // rows still to visit, per bank, over the whole domain
+    for (int l = 0; l < 32; ++l) {
+        if ((int)d.rows[l].size() != n) return false;
+        for (int i = 1; i < n; ++i)
+            if (d.rows[l][i] - d.rows[l][i - 1] > 127) return false;
+        for (int i = 0; i < n; ++i)
+            if (d.rows[l][i] < d.zero_row) ++demand[d.rows[l][i] & 31];
+        lane[l].seen.assign(n, 0);
+        d.order[l].assign(n, 0);
+    }
+    auto fits = [](int step) { return step >= -128 && step <= 127; };
+    // Kuhn's augmenting paths, lanes to banks, every bank taking up to `cap` lanes
+    struct Matcher {
+        Lane *lane;
+        RunDomain &d;
+        int cap = 1;
+        int owners[32][32], count[32];
+        bool tried[32];
+        bool place(int l)
+        {
+            for (int i : lane[l].cand) {
+                const int row = d.rows[l][i];
+                if (row >= d.zero_row) {  // padding: every lane's padding is the same address
+                    lane[l].pick = i;
+                    return true;
+                }
+                const int b = row & 31;
+                if (tried[b]) continue;
+                tried[b] = true;
+                if (count[b] < cap) {
+                    owners[b][count[b]++] = l;
+                    lane[l].pick = i;
+                    return true;
+                }
+                for (int k = 0; k < count[b]; ++k)
+                    if (place(owners[b][k])) {
+                        owners[b][k] = l;
+                        lane[l].pick = i;
+                        return true;
+                    }
+            }
+            return false;
+        }
+    } m{lane, d};
+
+    double credit = 0.0;
+    for (int step = 0; step < n; ++step) {
+        // A bank asked for more often than there are steps left has to be served more than once
+        // per step at some point; doing that at an even rate costs the fewest passes overall.
+        double q = 1.0;
+        for (int b = 0; b < 32; ++b) q = std::max(q, (double)demand[b] / (n - step));
+        credit += q;
+        const int cap = std::max(1, (int)credit);  // e.g. q = 1.3: one step in three serves every bank twice
+        credit -= cap;
+        for (int l = 0; l < 32; ++l) {
+            Lane &L = lane[l];
+            const std::vector<uint16_t> &r = d.rows[l];
+            L.cand.clear();
+            L.pick = -1;
+            int prev = -1;  // last unvisited entry before i
+            for (int i = L.lo, taken = 0; i < n && taken < window; ++i) {
+                if (L.seen[i]) continue;
+                ++taken;
+                int next = i + 1;
+                while (next < n && L.seen[next]) ++next;
+                // a pick must be in reach, must leave its unvisited neighbours in reach of each other,
+                // and must leave the oldest unvisited entry in reach of itself
+                bool ok = L.cur < 0 || fits(r[i] - L.cur);
+                if (ok && prev >= 0 && next < n) ok = fits(r[next] - r[prev]);
+                const int lo2 = i == L.lo ? next : L.lo;
+                if (ok && lo2 < n) ok = fits(r[lo2] - r[i]);
+                if (ok) L.cand.push_back(i);
+                prev = i;
+            }
+            if (L.cand.empty()) return false;  // cannot happen while the sorted gaps fit; kept as a guard
+            std::stable_sort(L.cand.begin(), L.cand.end(), [&](int x, int y) {
+                const int dx = r[x] >= d.zero_row ? -1 : demand[r[x] & 31], dy = r[y] >= d.zero_row ? -1 : demand[r[y] & 31];
+                return dx > dy;
+            });
+        }
+        m.cap = cap;
+        for (int b = 0; b < 32; ++b) m.count[b] = 0;
+        int load[32] = {0};
+        bool placed[32];
+        for (int l = 0; l < 32; ++l) {
+            for (int b = 0; b < 32; ++b) m.tried[b] = false;
+            placed[l] = m.place(l);
+        }
+        for (int b = 0; b < 32; ++b) load[b] = m.count[b];
+        for (int l = 0; l < 32; ++l) {
+            Lane &L = lane[l];
+            if (!placed[l]) {  // no bank with room: join the least loaded one
+                int best = L.cand[0];
+                for (int i : L.cand)
+                    if (load[d.rows[l][i] & 31] < load[d.rows[l][best] & 31]) best = i;
+                L.pick = best;
+                ++load[d.rows[l][best] & 31];
+            }
+            L.seen[L.pick] = 1;
+            L.cur = d.rows[l][L.pick];
+            if (L.cur < d.zero_row) --demand[L.cur & 31];
+            d.order[l][step] = (uint16_t)L.cur;
+            while (L.lo < n && L.seen[L.lo]) ++L.lo;
+        }
+    }
+    return true;
+}
+
 int u16_index_shift(int K) { return 4 * K <= 65535 ? 2 : 0; }
 int ragged_index_shift(int K) { return 4 * (K + 64) <= 65536 ? 2 : 0; }
 
@@ -381,9 +498,12 @@ int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint1
 }
 
 // ---------------------------------------------------------------- gap streams
-// Task layout: 256-byte header of restart indices, u16 [sign][lane], then the
-// gap rounds.  The first gap of every run is stored as 0 (the restart index is
-// the run's first row), so a lane's walk is "idx = restart; idx += gap; gather".
+// Task layout: 256-byte header of first rows, u16 [sign][lane], then the gap
+// rounds.  The first gap of every lane is stored as 0 (the header holds the first
+// row), so a lane's walk is "row = first; row += gap; gather".  A lane owns a
+// contiguous run of the sorted list.  16-bit gaps are unsigned and follow the
+// sorted order; 8-bit gaps are signed and follow the order schedule_runs() picks,
+// which keeps the lanes of a half-wavefront on different LDS banks.
 int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int split_k)
 {
     Geometry g;
@@ -396,7 +516,7 @@ int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int
                 if (i % g.n_lane == 0) continue;  // run start: absolute
                 size_t o = (size_t)c * g.half + i;
                 if (l[o] <= l[o - 1]) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending");
-                if (l[o] - l[o - 1] > 255) return 16;
+                if (l[o] - l[o - 1] > 127) return 16;
             }
     }
     return 8;
@@ -410,6 +530,33 @@ size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits)
     return (size_t)g.tasks * (256 + (size_t)64 * 2 * g.n_lane * (bits / 8));
 }
 
+}  // extern "C"
+
+namespace sptmm {
+
+bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint16_t> (&rows)[2][64])
+{
+    for (int sign = 0; sign < 2; ++sign)
+        for (int h = 0; h < 2; ++h) {
+            RunDomain d;
+            d.n = n;
+            d.zero_row = zero_row;
+            for (int l = 0; l < 32; ++l) d.rows[l] = rows[sign][32 * h + l];
+            if (!schedule_runs(d)) return false;
+            for (int l = 0; l < 32; ++l) {
+                const int lane = 32 * h + l;
+                *(uint16_t *)(task + sign * 128 + lane * 2) = d.order[l][0];
+                for (int j = 0; j < n; ++j)
+                    task[256 + slot_offset(n, 1, sign, lane, j)] = (uint8_t)(int8_t)(j ? (int)d.order[l][j] - (int)d.order[l][j - 1] : 0);
+            }
+        }
+    return true;
+}
+
+}  // namespace sptmm
+
+extern "C" {
+
 static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int K, int N, int S, int split_k, int bits)
 {
     if (int rc = check_shape(K, N, S)) return rc;
@@ -421,10 +568,29 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
     const size_t task_bytes = 256 + (size_t)128 * g.n_lane * esz;
     uint8_t *base = (uint8_t *)packed;
     std::vector<int> bad(N, 0);
+    if (pack && bits == 8) {
+        for (int sign = 0; sign < 2; ++sign) {
+            const uint16_t *l = sign ? neg : pos;
+            for (size_t i = 1, e = (size_t)N * g.half; i < e; ++i)
+                if (i % g.n_lane && l[i] <= l[i - 1]) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending");
+        }
+        parallel_columns(g.tasks, [&](int t) {
+            std::vector<uint16_t> rows[2][64];
+            for (int sign = 0; sign < 2; ++sign)
+                for (int lane = 0; lane < 64; ++lane) {
+                    const uint16_t *lst = (sign ? neg : pos) + (size_t)(t * g.G + lane / g.L) * g.half + (size_t)(lane % g.L) * g.n_lane;
+                    rows[sign][lane].assign(lst, lst + g.n_lane);
+                }
+            if (!write_task_runs8(base + (size_t)t * task_bytes, g.n_lane, K, rows)) bad[t * g.G] = 1;
+        });
+        for (int c = 0; c < N; ++c)
+            if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d: a gap does not fit 8 bits (signed)", c);
+        return SPTMM_OK;
+    }
     parallel_columns(N, [&](int c) {
         for (int sign = 0; sign < 2; ++sign) {
             uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
-            unsigned run = 0;
+            int run = 0;
             for (int i = 0; i < g.half; ++i) {
                 Place p = place(g, c, i, true);
                 uint8_t *task = base + p.task * task_bytes;
@@ -436,22 +602,24 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
                         *restart = lst[i];
                     } else {
                         gap = (unsigned)lst[i] - lst[i - 1];
-                        if (lst[i] <= lst[i - 1] || gap >= (1u << bits)) bad[c] = 1;
+                        if (lst[i] <= lst[i - 1]) bad[c] = 1;
                     }
                     if (esz == 1)
                         *cell = (uint8_t)gap;
                     else
                         *(uint16_t *)cell = (uint16_t)gap;
                 } else {
-                    unsigned gap = esz == 1 ? *cell : *(uint16_t *)cell;
+                    const int gap = esz == 1 ? (int)(int8_t)*cell : (int)*(uint16_t *)cell;
                     run = p.slot == 0 ? *restart + gap : run + gap;
+                    if (run < 0 || run >= K) bad[c] = 1;
                     lst[i] = (uint16_t)run;
                 }
             }
+            if (!pack) std::sort(lst, lst + g.half);  // 8-bit streams visit a run in scheduled order
         }
     });
     for (int c = 0; c < N; ++c)
-        if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d: list not ascending or gap does not fit %d bits", c, bits);
+        if (bad[c]) return fail(SPTMM_ERR_INVALID, pack ? "column %d: list not ascending" : "column %d: corrupt gap stream", c);
     return SPTMM_OK;
 }
 

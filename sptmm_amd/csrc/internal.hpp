@@ -52,6 +52,25 @@ struct Domain {
 };
 void schedule(Domain &d);
 
+// Gap streams with 8-bit gaps store them SIGNED, so a lane may visit the rows of
+// its run in any order whose steps stay within -128..127.  schedule_runs() picks
+// those orders for the 32 lanes of a half-wavefront together: at every step each
+// lane chooses among the oldest `window` rows it has not visited yet, and the
+// choices are matched to distinct LDS banks (row mod 32) as far as possible.
+// rows[l]: ascending, all of the same length n; rows >= zero_row are padding (the
+// same zero slot for every lane, never a conflict).  order[l][j] = row that lane l
+// visits at step j.  Returns false when some run has a sorted gap above 127 (no
+// 8-bit stream exists then).
+struct RunDomain {
+    int n = 0, zero_row = 0;
+    std::vector<uint16_t> rows[32];
+    std::vector<uint16_t> order[32];
+};
+bool schedule_runs(RunDomain &d, int window = 8);
+// One task of an 8-bit gap stream (header + rounds at `task`): rows[sign][lane] = what the lane
+// visits, ascending, n each.  False when a sorted gap exceeds 127.
+bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint16_t> (&rows)[2][64]);
+
 // Geometry of a ragged stream (tasks carry their own entry count): as
 // make_geometry, with half = n_lane = 0.
 int make_ragged_geometry(int N, int split_k, int max_split, Geometry *g);

@@ -59,8 +59,9 @@ __device__ __forceinline__ void gather(const unsigned char *lds, u32 addr, typen
 
 // Stream flavours (MODE):
 //   0  u16 row indices (already multiplied by 4 when PRE)
-//   1  8-bit gaps in rows, contiguous run per lane (256-byte task header: first row of every lane and sign)
-//   2  the same with 16-bit gaps
+//   1  signed 8-bit gaps in rows; each lane walks a contiguous run of the sorted list in the
+//      order the host scheduled (256-byte task header: first row of every lane and sign)
+//   2  unsigned 16-bit gaps, runs walked in ascending order
 // VAR (template flag of the kernels): ragged tasks.  The stream starts with a
 // table of per-task entry counts and the tasks sit at a fixed stride; lists
 // shorter than their task's count are padded with entries on the zero rows
@@ -82,7 +83,7 @@ __device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &ru
     if constexpr (Flavour<MODE>::GAP8) {
 #pragma unroll
         for (int b = 0; b < NBYTES; ++b) {
-            run += ((d >> (8 * b)) & 0xffu) << SH;
+            run += (u32)((int)(d << (24 - 8 * b)) >> 24) << SH;  // signed gap
             gather<Act, MT, NEG>(lds, run, acc);
         }
     } else {

@@ -125,10 +125,10 @@ int ragged_plan(const int8_t *W, int K, int N, int kind, int split_k, int bits_r
                 const std::vector<uint16_t> &e = pl->rows[sign][c];
                 const int n = pl->n_task[c / g.G], cnt = (int)e.size();
                 for (int i = 1; i < cnt; ++i)
-                    if (i % n && e[i] - e[i - 1] > 255) fits8 = false;
-                if (cnt % n && K - e[cnt - 1] > 255) fits8 = false;
+                    if (i % n && e[i] - e[i - 1] > 127) fits8 = false;
+                if (cnt % n && K - e[cnt - 1] > 127) fits8 = false;
             }
-        if (bits_req == 8 && !fits8) return fail(SPTMM_ERR_UNSUPPORTED, "a gap does not fit 8 bits");
+        if (bits_req == 8 && !fits8) return fail(SPTMM_ERR_UNSUPPORTED, "a gap does not fit 8 bits (signed)");
         pl->bits = bits_req ? bits_req : (fits8 ? 8 : 16);
         pl->esz = pl->bits / 8;
         pl->hdr = 256;
@@ -207,32 +207,34 @@ void pack_u16(const RaggedPlan &pl, uint8_t *stream)
     put_counts(pl, stream);
 }
 
-// Lane v of a column walks entries [v*n, (v+1)*n) of the sorted list; where the list ends the lane
-// steps to the zero row K and stays there (gap 0), and the lanes behind it start on K.
+// Lane v of a column owns entries [v*n, (v+1)*n) of the sorted list; where the list ends the lane
+// steps to the zero row K and stays there (gap 0), and the lanes behind it start on K.  16-bit
+// gaps follow the sorted order; 8-bit gaps are signed and follow the bank-aware order.
 void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
 {
     const Geometry &g = pl.g;
     uint8_t *base = stream + pl.counts_bytes;
-    parallel_for(g.N, [&](int c) {
-        const int task = c / g.G, l0 = (c % g.G) * g.L, n = pl.n_task[task];
+    parallel_for(g.tasks, [&](int task) {
+        const int n = pl.n_task[task];
         uint8_t *t = base + (size_t)task * pl.stride;
-        for (int sign = 0; sign < 2; ++sign) {
-            const std::vector<uint16_t> &e = pl.rows[sign][c];
-            const int cnt = (int)e.size();
-            for (int v = 0; v < g.L; ++v) {
-                const int lane = l0 + v, first = v * n;
-                int prev = first < cnt ? e[first] : pl.K;
-                *(uint16_t *)(t + sign * 128 + lane * 2) = (uint16_t)prev;
-                for (int i = 0; i < n; ++i) {
-                    const int row = first + i < cnt ? e[first + i] : pl.K;
-                    uint8_t *cell = t + pl.hdr + slot_offset(n, pl.esz, sign, lane, i);
-                    if (pl.esz == 1)
-                        *cell = (uint8_t)(row - prev);
-                    else
-                        *(uint16_t *)cell = (uint16_t)(row - prev);
-                    prev = row;
-                }
+        std::vector<uint16_t> rows[2][64];
+        for (int sign = 0; sign < 2; ++sign)
+            for (int lane = 0; lane < 64; ++lane) {
+                const std::vector<uint16_t> &e = pl.rows[sign][task * g.G + lane / g.L];
+                const int cnt = (int)e.size(), first = (lane % g.L) * n;
+                std::vector<uint16_t> &r = rows[sign][lane];
+                r.resize(n);
+                for (int i = 0; i < n; ++i) r[i] = first + i < cnt ? e[first + i] : (uint16_t)pl.K;
             }
+        if (pl.esz == 1) {
+            write_task_runs8(t, n, pl.K, rows);  // the plan has checked that every gap fits
+        } else {
+            for (int sign = 0; sign < 2; ++sign)
+                for (int lane = 0; lane < 64; ++lane) {
+                    const std::vector<uint16_t> &r = rows[sign][lane];
+                    *(uint16_t *)(t + sign * 128 + lane * 2) = r[0];
+                    for (int i = 0; i < n; ++i) *(uint16_t *)(t + pl.hdr + slot_offset(n, 2, sign, lane, i)) = (uint16_t)(i ? r[i] - r[i - 1] : 0);
+                }
         }
     });
     put_counts(pl, stream);
@@ -340,9 +342,12 @@ int sptmm_unpack_ragged(const void *packed, int K, int N, int kind, int split_k,
                     int row = gaps ? *(const uint16_t *)(t + sign * 128 + lane * 2) : 0;
                     for (int i = 0; i < (int)n; ++i) {
                         const uint8_t *cell = t + hdr + slot_offset((int)n, esz, sign, lane, i);
-                        const int f = esz == 1 ? *cell : *(const uint16_t *)cell;
+                        const int f = esz == 1 ? (gaps ? (int)(int8_t)*cell : (int)*cell) : (int)*(const uint16_t *)cell;
                         row = gaps ? row + f : f >> sh;
-                        if (row >= K + 64) bad[task] = 1;
+                        if (row < 0 || row >= K + 64) {
+                            bad[task] = 1;
+                            continue;
+                        }
                         if (row >= K) continue;  // padding
                         int8_t &w = W[(size_t)col * K + row];
                         if (w) bad[task] = 1;  // a row may appear once per column

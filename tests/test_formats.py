@@ -137,7 +137,7 @@ def test_delta_stream_round_trips(K, N, S, split):
     gaps_fit = True
     for lst in (pos, neg):
         runs = lst.reshape(N, split, n_lane).astype(int)
-        gaps_fit &= bool((np.diff(runs, axis=2) <= 255).all())
+        gaps_fit &= bool((np.diff(runs, axis=2) <= 127).all())  # 8-bit gaps are signed
     assert bits == (8 if gaps_fit else 16)
     pk, b = sp.pack_delta(pos, neg, K, split)
     assert b == bits and pk.nbytes == N // (64 // split) * (256 + 128 * n_lane * bits // 8)
@@ -155,29 +155,94 @@ def test_delta_8bit_refuses_wide_gaps():
     assert sp.delta_bits(pos, neg, 8) == 16
     with pytest.raises(sp.SptmmError):
         sp.pack_delta(pos, neg, K, 8, bits=8)
+    # a gap of 128 no longer fits the signed byte, 127 does
+    for gap, want in ((127, 8), (128, 16)):
+        pos = np.tile(np.arange(8, dtype=np.uint16), (16, 1))
+        pos[:, 1:] += gap - 1
+        neg = pos + 300
+        assert sp.delta_bits(pos, neg, 8) == 8  # one entry per lane: no in-run gap at all
+        assert sp.delta_bits(np.ascontiguousarray(np.repeat(pos, 2, 1)[:, :16] + np.arange(16, dtype=np.uint16) % 2 * gap),
+                             np.ascontiguousarray(np.repeat(neg, 2, 1)[:, :16] + np.arange(16, dtype=np.uint16) % 2 * gap), 8) == want
 
 
-def test_delta_gaps_match_oracle_within_runs():
-    # inside a run the stored bytes are the reference's gaps (main.cu:376-394)
-    K, N, S, split = 2560, 16, 1536, 32
+def lane_walk(task, n_lane, esz, sign, lane):
+    """Rows one lane visits, in order: first row from the header, then the (signed 8-bit / unsigned 16-bit) gaps."""
+    first = int(task[sign * 128 + 2 * lane: sign * 128 + 2 * lane + 2].view(np.uint16)[0])
+    off = [256 + slot_offset(n_lane, esz, sign, lane, j) for j in range(n_lane)]
+    if esz == 1:
+        gaps = task[off].view(np.int8).astype(int)
+    else:
+        gaps = np.array([int(task[o:o + 2].view(np.uint16)[0]) for o in off])
+    assert gaps[0] == 0
+    return first + np.cumsum(gaps)
+
+
+def slot_offset(n_lane, esz, sign, lane, j):
+    e16 = 16 // esz
+    full = n_lane // e16
+    if j < full * e16:
+        return (j // e16) * 2048 + sign * 1024 + lane * 16 + (j % e16) * esz
+    base, rem, first = full * 2048, n_lane - full * e16, full * e16
+    w = 8
+    while w >= esz:
+        cnt = w // esz
+        if rem & cnt:
+            if j < first + cnt:
+                return base + sign * 64 * w + lane * w + (j - first) * esz
+            first += cnt
+            base += 128 * w
+        w //= 2
+    raise AssertionError
+
+
+@pytest.mark.parametrize("K,N,S,split", [(2560, 16, 1536, 32), (6912, 16, 4096, 64), (6912, 16, 4160, 16), (2560, 16, 1536, 8)])
+def test_delta_8bit_lanes_walk_their_own_run_in_a_bank_friendly_order(K, N, S, split):
+    """Each lane visits exactly the contiguous run of the sorted list the reference's gaps describe
+    (main.cu:376-394: gap i = row i - row i-1), in an order whose steps fit a signed byte, and the 32
+    lanes of a half-wavefront mostly sit on 32 different banks (row mod 32)."""
     _, pos, neg = sp.generate_ternary(K, N, S)
     d_ref, wrapped = oracle.delta8(pos)
     assert wrapped == 0
     pk, bits = sp.pack_delta(pos, neg, K, split)
     assert bits == 8
-    n_lane = (S // 2) // split  # 24 = one 16-byte round + one 8-byte round
+    L, G = min(split, 64), 64 // min(split, 64)
+    n_lane = (S // 2) // split
     task_bytes = 256 + 128 * n_lane
-    for c in (0, 3, 15):
-        for v in (0, 5, 31):
-            lane = (c % 2) * 32 + v
-            t = pk[(c // 2) * task_bytes:(c // 2 + 1) * task_bytes]
-            restart = t[:256].view(np.uint16)[lane]
-            assert restart == pos[c, v * n_lane]
-            got = np.concatenate([t[256 + lane * 16: 256 + lane * 16 + 16],
-                                  t[256 + 2048 + lane * 8: 256 + 2048 + lane * 8 + 8]])
-            want = d_ref[c, v * n_lane:(v + 1) * n_lane].copy()
-            want[0] = 0
-            assert (got == want).all()
+    passes = slots = 0
+    for t in range(N // G):
+        task = pk[t * task_bytes:(t + 1) * task_bytes]
+        for sign, lst in ((0, pos), (1, neg)):
+            walks = []
+            for lane in range(64):
+                c, v = t * G + lane // L, lane % L
+                w = lane_walk(task, n_lane, 1, sign, lane)
+                run = lst[c, v * n_lane:(v + 1) * n_lane].astype(int)
+                assert sorted(w) == list(run)
+                assert np.abs(np.diff(w)).max(initial=0) <= 128
+                if sign == 0 and n_lane > 1:  # the sorted run's gaps are the reference's delta bytes
+                    assert (np.diff(run) == d_ref[c, v * n_lane + 1:(v + 1) * n_lane]).all()
+                walks.append(w)
+            walks = np.array(walks)
+            for h in range(2):
+                for j in range(n_lane):
+                    passes += np.bincount(walks[32 * h:32 * h + 32, j] & 31, minlength=32).max()
+                    slots += 1
+    # sorted order needs ~3.5 passes per step; the schedule must stay well below 2
+    assert passes <= 1.45 * slots, (passes / slots)
+
+
+def test_delta_16bit_follows_sorted_order():
+    K, N, S, split = 6912, 16, 256, 8
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    pk, bits = sp.pack_delta(pos, neg, K, split)
+    assert bits == 16
+    n_lane = (S // 2) // split
+    task_bytes = 256 + 256 * n_lane
+    for c in (0, 9):
+        task = pk[(c // 8) * task_bytes:(c // 8 + 1) * task_bytes]
+        for v in (0, 7):
+            w = lane_walk(task, n_lane, 2, 1, (c % 8) * 8 + v)
+            assert (w == neg[c, v * n_lane:(v + 1) * n_lane]).all()
 
 
 def test_i2s_word_and_stream():

@@ -118,11 +118,13 @@ def test_sizes_and_counts_closed_form(split):
         assert (packed[16:16 + 2 * tasks].view(np.uint16) == n_task).all() and not packed[16 + 2 * tasks:table].any()
 
 
-def test_gap_stream_cells_follow_the_documented_walk():
-    """Lane v holds entries [v*n, (v+1)*n) of the sorted list as gaps; past the end it steps to row K and stays."""
+def test_gap_stream_lanes_visit_their_run_then_the_zero_row():
+    """Lane v holds entries [v*n, (v+1)*n) of the sorted list, visited in a scheduled order with signed
+    8-bit steps; past the end of the list it steps to row K and stays."""
     K, N, split = 512, 16, 16
     W = sp.generate_ternary_iid(K, N, 33, 0.3, 0.2)
     packed, inf = sp.pack_ragged(W, DELTA, split)
+    assert inf["bits"] == 8
     G, L = 64 // split, split
     stride, table = 256 + 128 * inf["n_max"], 256
     for c in (0, 5, 15):
@@ -134,9 +136,9 @@ def test_gap_stream_cells_follow_the_documented_walk():
                 lane = (c % G) * L + v
                 want = list(rows[v * n:(v + 1) * n]) + [K] * (n - len(rows[v * n:(v + 1) * n]))
                 first = int(task[sign * 128 + 2 * lane: sign * 128 + 2 * lane + 2].view(np.uint16)[0])
-                gaps = [int(task[256 + slot_offset(n, 1, sign, lane, j)]) for j in range(n)]
-                assert first == want[0] and gaps[0] == 0
-                assert list(first + np.cumsum(gaps)) == want
+                gaps = task[[256 + slot_offset(n, 1, sign, lane, j) for j in range(n)]].view(np.int8).astype(int)
+                walk = first + np.cumsum(gaps)
+                assert gaps[0] == 0 and sorted(walk) == want
 
 
 def test_sparse_matrix_takes_16_bit_gaps_and_8_bit_request_fails():
