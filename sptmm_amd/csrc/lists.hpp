@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <type_traits>
 
 #include "internal.hpp"
 
@@ -34,28 +35,82 @@ __host__ __device__ constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v
 
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 
-// acc[m] (+|-)= X[m][k] for the slot at byte offset `addr` of the tile
-template <typename Act, int MT, bool NEG>
-__device__ __forceinline__ void gather(const unsigned char *lds, u32 addr, typename Acc<Act>::type (&acc)[MT])
-{
-    if constexpr (sizeof(Act) == 1 && MT == 1) {
-        int v = *reinterpret_cast<const int *>(lds + addr);
-        acc[0] = NEG ? acc[0] - v : acc[0] + v;
-    } else if constexpr (sizeof(Act) == 1) {
-        Vec<int, MT / 4> r = *reinterpret_cast<const Vec<int, MT / 4> *>(lds + addr);
+// The running sums of one lane: acc[m] (+|-)= X[m][k] for every gathered row k.
+// int8 activations with MT > 1 keep the tile's bytes biased by 128 (unsigned) and
+// add them four rows at a time into 16-bit fields of plain 32-bit registers --
+// two masks, a shift and two adds per four rows, all in the short VOP2 encoding,
+// against four dot4 instructions (measured on gfx950: a VOP3 instruction costs
+// about twice a VOP2 one).  A field holds at most 257 entries (257 * 255 < 65536);
+// flush() widens the fields into acc[] and has to be called at least that often.
+// Both signs of a lane always gather the same number of entries, so the bias cancels.
+template <typename Act, int MT> struct Sums {
+    typedef typename Acc<Act>::type A;
+    static constexpr bool SWAR = sizeof(Act) == 1 && MT > 1;
+    static constexpr int NW = SWAR ? MT / 4 : 1;
+    A acc[MT];
+    u32 lo[2][NW], hi[2][NW];  // [sign][dword]: rows 4j / 4j+2 and rows 4j+1 / 4j+3 (SWAR only)
+
+    __device__ __forceinline__ void init()
+    {
 #pragma unroll
-        for (int m = 0; m < MT; ++m)  // dot4 with a one-hot (+1 or -1) selector: no unpacking
-            acc[m] = __builtin_amdgcn_sdot4(r.v[m / 4], (NEG ? 0xff : 0x01) << (8 * (m % 4)), acc[m], false);
-    } else if constexpr (sizeof(Act) == 2 && MT > 1) {
-        Vec<_Float16, MT> r = *reinterpret_cast<const Vec<_Float16, MT> *>(lds + addr);
+        for (int m = 0; m < MT; ++m) acc[m] = (A)0;
+        if constexpr (SWAR) {
 #pragma unroll
-        for (int m = 0; m < MT; ++m) acc[m] = NEG ? acc[m] - (float)r.v[m] : acc[m] + (float)r.v[m];
-    } else {
-        Vec<float, MT> r = *reinterpret_cast<const Vec<float, MT> *>(lds + addr);
-#pragma unroll
-        for (int m = 0; m < MT; ++m) acc[m] = NEG ? acc[m] - r.v[m] : acc[m] + r.v[m];
+            for (int j = 0; j < NW; ++j) lo[0][j] = hi[0][j] = lo[1][j] = hi[1][j] = 0u;
+        }
     }
-}
+
+    // What one slot of the tile holds (all MT rows of one index), as read from LDS.
+    typedef typename std::conditional<sizeof(Act) == 1, Vec<u32, NW>,
+                                      typename std::conditional<sizeof(Act) == 2 && (MT > 1), Vec<_Float16, MT>, Vec<float, MT>>::type>::type Raw;
+
+    // the slot at byte offset `addr` of the tile
+    static __device__ __forceinline__ Raw load(const unsigned char *lds, u32 addr) { return *reinterpret_cast<const Raw *>(lds + addr); }
+
+    template <bool NEG> __device__ __forceinline__ void accum(const Raw &r)
+    {
+        if constexpr (sizeof(Act) == 1 && MT == 1) {
+            acc[0] = NEG ? acc[0] - (int)r.v[0] : acc[0] + (int)r.v[0];
+        } else if constexpr (SWAR) {
+#pragma unroll
+            for (int j = 0; j < NW; ++j) {
+                lo[NEG][j] += r.v[j] & 0x00ff00ffu;
+                hi[NEG][j] += (r.v[j] >> 8) & 0x00ff00ffu;
+            }
+        } else {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) acc[m] = NEG ? acc[m] - (float)r.v[m] : acc[m] + (float)r.v[m];
+        }
+    }
+
+    // Pin the sums once per round.  Integer adds may be reassociated freely, and without
+    // this the compiler keeps every gathered value of every round alive to sum them in
+    // one tree at the end.
+    __device__ __forceinline__ void pin()
+    {
+        if constexpr (SWAR) {
+#pragma unroll
+            for (int j = 0; j < NW; ++j) asm volatile("" : "+v"(lo[0][j]), "+v"(hi[0][j]), "+v"(lo[1][j]), "+v"(hi[1][j]));
+        } else {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) asm volatile("" : "+v"(acc[m]));
+        }
+    }
+
+    __device__ __forceinline__ void flush()
+    {
+        if constexpr (SWAR) {
+#pragma unroll
+            for (int j = 0; j < NW; ++j) {
+                acc[4 * j + 0] += (int)(lo[0][j] & 0xffffu) - (int)(lo[1][j] & 0xffffu);
+                acc[4 * j + 1] += (int)(hi[0][j] & 0xffffu) - (int)(hi[1][j] & 0xffffu);
+                acc[4 * j + 2] += (int)(lo[0][j] >> 16) - (int)(lo[1][j] >> 16);
+                acc[4 * j + 3] += (int)(hi[0][j] >> 16) - (int)(hi[1][j] >> 16);
+                lo[0][j] = hi[0][j] = lo[1][j] = hi[1][j] = 0u;
+            }
+        }
+    }
+};
 
 // Stream flavours (MODE):
 //   0  u16 row indices (already multiplied by 4 when PRE)
@@ -74,17 +129,40 @@ template <int MODE> struct Flavour {
 };
 constexpr int RAGGED_PREAMBLE = 16;  // {magic, tasks, n_max, n_min} in front of the u16 count table
 
-// `run` is the byte offset of the current row's slot in the tile.  Consumes the
-// low NBYTES of `d`.
-template <typename Act, int MT, int MODE, bool PRE, bool NEG, int NBYTES>
-__device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &run, typename Acc<Act>::type (&acc)[MT])
+// run += sign-extended byte B of d, in one SDWA add
+template <int B> __device__ __forceinline__ void add_signed_byte(u32 &run, u32 d)
 {
+    if constexpr (B == 0)
+        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:DWORD" : "+v"(run) : "v"(d));
+    else if constexpr (B == 1)
+        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:DWORD" : "+v"(run) : "v"(d));
+    else if constexpr (B == 2)
+        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2 src1_sel:DWORD" : "+v"(run) : "v"(d));
+    else
+        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3 src1_sel:DWORD" : "+v"(run) : "v"(d));
+}
+
+// `run` is the current row of a gap stream: the row index itself with 8-bit gaps,
+// the byte offset of the row's slot in the tile with 16-bit gaps.  fetch() turns
+// the low NBYTES of `d` into tile reads (all of them issued before anything is
+// added up, so a round keeps its 16 or 32 LDS reads in flight together).
+template <typename Act, int MT, int MODE, bool PRE, int NBYTES>
+__device__ __forceinline__ void fetch(const unsigned char *lds, u32 d, u32 &run, typename Sums<Act, MT>::Raw *r)
+{
+    typedef Sums<Act, MT> S;
     constexpr int SH = ilog2(slot_bytes<Act, MT>());
     if constexpr (Flavour<MODE>::GAP8) {
-#pragma unroll
-        for (int b = 0; b < NBYTES; ++b) {
-            run += (u32)((int)(d << (24 - 8 * b)) >> 24) << SH;  // signed gap
-            gather<Act, MT, NEG>(lds, run, acc);
+        add_signed_byte<0>(run, d);
+        r[0] = S::load(lds, run << SH);
+        if constexpr (NBYTES > 1) {
+            add_signed_byte<1>(run, d);
+            r[1] = S::load(lds, run << SH);
+        }
+        if constexpr (NBYTES > 2) {
+            add_signed_byte<2>(run, d);
+            r[2] = S::load(lds, run << SH);
+            add_signed_byte<3>(run, d);
+            r[3] = S::load(lds, run << SH);
         }
     } else {
 #pragma unroll
@@ -92,21 +170,35 @@ __device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &ru
             u32 f = h ? (d >> 16) : (d & 0xffffu);
             if constexpr (Flavour<MODE>::GAP16) {
                 run += f << SH;
-                gather<Act, MT, NEG>(lds, run, acc);
+                r[h] = S::load(lds, run);
             } else {
-                gather<Act, MT, NEG>(lds, f << (PRE ? SH - 2 : SH), acc);
+                r[h] = S::load(lds, f << (PRE ? SH - 2 : SH));
             }
         }
     }
 }
 
-template <typename Act, int MT, int MODE, bool PRE, bool NEG>
-__device__ __forceinline__ void consume16(const unsigned char *lds, const uint4 &v, u32 &run, typename Acc<Act>::type (&acc)[MT])
+template <typename Act, int MT, int MODE, bool PRE, bool NEG, int NBYTES>
+__device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &run, Sums<Act, MT> &acc)
 {
-    consume<Act, MT, MODE, PRE, NEG, 4>(lds, v.x, run, acc);
-    consume<Act, MT, MODE, PRE, NEG, 4>(lds, v.y, run, acc);
-    consume<Act, MT, MODE, PRE, NEG, 4>(lds, v.z, run, acc);
-    consume<Act, MT, MODE, PRE, NEG, 4>(lds, v.w, run, acc);
+    constexpr int NE = NBYTES / Flavour<MODE>::ESZ;
+    typename Sums<Act, MT>::Raw r[NE];
+    fetch<Act, MT, MODE, PRE, NBYTES>(lds, d, run, r);
+#pragma unroll
+    for (int e = 0; e < NE; ++e) acc.template accum<NEG>(r[e]);
+}
+
+template <typename Act, int MT, int MODE, bool PRE, bool NEG>
+__device__ __forceinline__ void consume16(const unsigned char *lds, const uint4 &v, u32 &run, Sums<Act, MT> &acc)
+{
+    constexpr int NE = 4 / Flavour<MODE>::ESZ;  // entries per dword
+    typename Sums<Act, MT>::Raw r[4 * NE];
+    fetch<Act, MT, MODE, PRE, 4>(lds, v.x, run, r);
+    fetch<Act, MT, MODE, PRE, 4>(lds, v.y, run, r + NE);
+    fetch<Act, MT, MODE, PRE, 4>(lds, v.z, run, r + 2 * NE);
+    fetch<Act, MT, MODE, PRE, 4>(lds, v.w, run, r + 3 * NE);
+#pragma unroll
+    for (int e = 0; e < 4 * NE; ++e) acc.template accum<NEG>(r[e]);
 }
 
 // 4 rows x 4 consecutive k (one dword per row) -> 4 dwords, dword j = the 4 rows at k+j
@@ -158,12 +250,13 @@ template <typename Act, int MT> struct Stager {
             for (int j = 0; j < 4; ++j) {
                 u32 o[4], q[4];
                 transpose4x4(comp(r[0], j), comp(r[1], j), comp(r[2], j), comp(r[3], j), o);
+                constexpr u32 B = 0x80808080u;  // bytes are stored biased by 128 (see Sums)
                 if constexpr (MT == 4) {
-                    t[4 * item + j] = make_uint4(o[0], o[1], o[2], o[3]);
+                    t[4 * item + j] = make_uint4(o[0] ^ B, o[1] ^ B, o[2] ^ B, o[3] ^ B);
                 } else {
                     transpose4x4(comp(r[4], j), comp(r[5], j), comp(r[6], j), comp(r[7], j), q);
-                    t[2 * (4 * item + j)] = make_uint4(o[0], q[0], o[1], q[1]);
-                    t[2 * (4 * item + j) + 1] = make_uint4(o[2], q[2], o[3], q[3]);
+                    t[2 * (4 * item + j)] = make_uint4(o[0] ^ B, q[0] ^ B, o[1] ^ B, q[1] ^ B);
+                    t[2 * (4 * item + j) + 1] = make_uint4(o[2] ^ B, q[2] ^ B, o[3] ^ B, q[3] ^ B);
                 }
             }
         } else if constexpr (sizeof(Act) == 2 && MT == 1) {  // 16 halves -> 16 floats
@@ -269,15 +362,11 @@ struct ListsBody {
 #endif
     static constexpr int EARLY = SPTMM_EARLY;         // rounds requested before the activation tile is complete
 
-    static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, A (&acc)[MT])
+    static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, Sums<Act, MT> &acc)
     {
         consume16<Act, MT, MODE, PRE, false>(smem, x.p, runp, acc);
         consume16<Act, MT, MODE, PRE, true>(smem, x.q, runq, acc);
-        // Pin the sums (and the running rows) once per round.  Integer adds may be
-        // reassociated freely, and without this the compiler keeps every gathered
-        // value of every round alive to sum them in one tree at the end.
-#pragma unroll
-        for (int m = 0; m < MT; ++m) asm volatile("" : "+v"(acc[m]));
+        acc.pin();  // (and the running rows)
         if constexpr (GAPS) asm volatile("" : "+v"(runp), "+v"(runq));
     }
 
@@ -349,7 +438,9 @@ struct ListsBody {
             St::load(X, p.M, p.K, m0, item, r);
             St::store(smem, item, r);
         }
-        for (int i = tid; i < ZROWS * SLOT / 4; i += nt) reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = 0u;  // rows K.. read as zero
+        // rows K.. read as zero (biased bytes: 128)
+        for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
+            reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = Sums<Act, MT>::SWAR ? 0x80808080u : 0u;
         __syncthreads();
 
         A *C = reinterpret_cast<A *>(p.C);
@@ -362,8 +453,8 @@ struct ListsBody {
             int n_lane = p.n_lane;
             if constexpr (GAPS) {
                 const unsigned short *rs = reinterpret_cast<const unsigned short *>(tb);
-                runp = (u32)rs[lane] << SH;
-                runq = (u32)rs[64 + lane] << SH;
+                runp = (u32)rs[lane] << (Fl::GAP8 ? 0 : SH);
+                runq = (u32)rs[64 + lane] << (Fl::GAP8 ? 0 : SH);
             }
             if constexpr (VAR) {
                 n_lane = __builtin_amdgcn_readfirstlane(n_ahead);
@@ -371,9 +462,8 @@ struct ListsBody {
                 n_ahead = counts[nxt < p.tasks ? nxt : 0];
             }
             const int R = n_lane / E16, rem = n_lane - R * E16;
-            A acc[MT];
-#pragma unroll
-            for (int m = 0; m < MT; ++m) acc[m] = (A)0;
+            Sums<Act, MT> acc;
+            acc.init();
 
             if constexpr (RF > 0) {
                 if (it > 0) {
@@ -434,6 +524,7 @@ struct ListsBody {
                         eat(smem, buf[i], runp, runq, acc);
                         buf[i] = load_round(wp, base + RING + i);
                     }
+                    acc.flush();  // at most 8 rounds = 128 entries per sign since the last one
                 }
                 if (R - base > RING) {
 #pragma unroll
@@ -443,6 +534,7 @@ struct ListsBody {
                         buf[i] = load_round(wp, r < R ? r : R - 1);
                     }
                     base += RING;
+                    acc.flush();
                 }
 #pragma unroll
                 for (int i = 0; i < RING; ++i) {
@@ -480,21 +572,22 @@ struct ListsBody {
                 }
             }
 
+            acc.flush();  // since the last one: at most 10 rounds and the tail, 175 entries per sign
 #pragma unroll
-            for (int m = 0; m < MT; ++m) acc[m] = lanes_sum(acc[m], p.logL);
+            for (int m = 0; m < MT; ++m) acc.acc[m] = lanes_sum(acc.acc[m], p.logL);
 
             if (p.W == 1) {
                 if (active && (lane & (L - 1)) == 0) {
                     const int col = (task << (6 - p.logL)) + (lane >> p.logL);
 #pragma unroll
                     for (int m = 0; m < MT; ++m)
-                        if (m0 + m < p.M) C[(size_t)(m0 + m) * p.N + col] = acc[m];
+                        if (m0 + m < p.M) C[(size_t)(m0 + m) * p.N + col] = acc.acc[m];
                 }
             } else {
                 // second pass: the W wavefronts of a column meet in a small LDS buffer
                 if (lane == 0) {
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) part[wave * MT + m] = acc[m];
+                    for (int m = 0; m < MT; ++m) part[wave * MT + m] = acc.acc[m];
                 }
                 __syncthreads();
                 if (active && lane == 0 && (wave & (p.W - 1)) == 0) {

@@ -90,6 +90,47 @@ def run_shape(name, K, N, S, Ms, splits, st, rows, iid=None):
                   flush=True)
 
 
+def layer_sequence(shapes, M, st, rows, iid=None):
+    """The layer's launches one after the other on one stream, each with its best split: plain launches and
+    one HIP graph per layer; cache-warm (one set of streams) and HBM-cold (rotating over 8 sets)."""
+    Kmax, Nmax = max(k for _, k, *_ in shapes), max(n for _, _, n, *_ in shapes)
+    xb = sp.DeviceBuffer.from_numpy(sp.make_x_i8(0xC0FFEE ^ M, M, Kmax))
+    cb = sp.DeviceBuffer(4 * M * Nmax)
+    for kind in ("u16", "delta", "i2s"):
+        layer, nbytes = [], 0
+        for name, K, N, S, mult in shapes:
+            best = min((r for r in rows if r["shape"] == name and r["M"] == M and r["enc"].startswith(kind)), key=lambda r: r["warm_us"])
+            split = int(best["enc"].split("/")[1]) if "/" in best["enc"] else 0
+            if iid is None:
+                W, pos, neg = sp.generate_ternary(K, N, S, dense=kind == "i2s")
+                w = (sp.Weights.upload_i2s(W) if kind == "i2s" else sp.Weights.upload_u16(pos, neg, K, split) if kind == "u16"
+                     else sp.Weights.upload_delta(pos, neg, K, split))
+            else:
+                W = sp.generate_ternary_iid(K, N, 0x5EED ^ N, *iid)
+                w = sp.Weights.upload_dense(W, {"u16": sp.KIND_U16, "delta": sp.KIND_DELTA, "i2s": sp.KIND_I2S}[kind], split or 32)
+            layer += [w] * mult
+            nbytes += mult * (w.info["stream_bytes"] + M * K + 4 * M * N)
+        sets = [layer] + [[w.clone() for w in layer] for _ in range(7)]
+        flat = [w for s_ in sets for w in s_]
+        out = {"shape": "layer_sequence", "M": M, "enc": kind, "launches": len(layer), "bytes": nbytes}
+        for label, ws in (("warm", layer), ("cold", flat)):
+            for mode, mname in ((0, "launches"), (2, "graph")):
+                sp.measure_gemv(ws, 0, xb, M, cb, 2 * len(ws), mode, st)
+                t = min(sp.measure_gemv(ws, 0, xb, M, cb, 40 * len(ws), mode, st) for _ in range(3)) * len(layer)
+                out["%s_%s_us" % (label, mname)] = round(t, 2)
+        print("layer in %d launches M=%d %-5s: warm %.1f us (graph %.1f)  cold %.1f us (graph %.1f; %.0f GB/s)"
+              % (len(layer), M, kind, out["warm_launches_us"], out["warm_graph_us"], out["cold_launches_us"], out["cold_graph_us"],
+                 nbytes / out["cold_graph_us"] / 1e3), flush=True)
+        rows.append(out)
+        for s_ in sets[1:]:
+            for w in s_:
+                w.free()
+        for w in set(layer):
+            w.free()
+    xb.free()
+    cb.free()
+
+
 def main(argv):
     which = argv[1] if len(argv) > 1 else "layer"
     info = sp.device_init(0)
@@ -110,6 +151,9 @@ def main(argv):
                 print("layer sum (%d launches, best split per shape) M=%d %-5s: warm %.1f us  cold %.1f us"
                       % (sum(m for *_, m in shapes), M, kind, tot_w, tot_c))
                 rows.append({"shape": "layer_sum", "M": M, "enc": kind, "warm_us": round(tot_w, 2), "cold_us": round(tot_c, 2)})
+        if which != "layer":
+            for M in (1, 4):
+                layer_sequence(shapes, M, st, rows, iid=(0.3, 0.3) if which == "ragged" else None)
     elif which == "large":
         run_shape("large", 13824, 5120, 8320, (1, 8, 16), (32, 64), st, rows)
     elif which == "headline":
