@@ -154,6 +154,13 @@ int sptmm_weights_upload_dense(const int8_t *W_colmajor, int K, int N, int kind,
  * the last-level cache holds when timing cold reads). */
 int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out);
 void sptmm_weights_free(sptmm_weights *w);
+/* Weight files, so that the host-side preparation (prepareW_map,
+ * main.cu:242-509, repeated by every run of the reference) happens once: a
+ * fixed header (shape, encoding, checksum) followed by the device stream as it
+ * is.  load checks the header against the stream size, the checksum and, for
+ * ragged streams, the count table, before anything reaches the device. */
+int sptmm_weights_save(const sptmm_weights *w, const char *path);
+int sptmm_weights_load(const char *path, sptmm_weights **out);
 int sptmm_weights_info(const sptmm_weights *w, sptmm_winfo *out);
 size_t sptmm_weights_bytes(const sptmm_weights *w);
 

@@ -27,7 +27,7 @@ EXPORTS = [
     "sptmm_unpack_ragged", "sptmm_generate_ternary_iid", "sptmm_dense_from_i2s_words", "sptmm_weights_upload_dense",
     "sptmm_device_init",
     "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
-    "sptmm_weights_upload_i2s", "sptmm_weights_clone",
+    "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
     "sptmm_gemv_f32", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
@@ -79,6 +79,8 @@ def lib() -> C.CDLL:
         L.sptmm_weights_bytes.argtypes = [C.c_void_p]
         L.sptmm_weights_info.argtypes = [C.c_void_p, C.POINTER(WInfo)]
         L.sptmm_weights_clone.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.sptmm_weights_save.argtypes = [C.c_void_p, C.c_char_p]
+        L.sptmm_weights_load.argtypes = [C.c_char_p, C.POINTER(C.c_void_p)]
         for n in ("sptmm_gemv_i8", "sptmm_gemv_f16", "sptmm_gemv_f32"):
             getattr(L, n).argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.sptmm_gemv_i8_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
@@ -385,6 +387,15 @@ class Weights:
         N, K = W.shape
         h = C.c_void_p()
         _ck(lib().sptmm_weights_upload_dense(_p(W), K, N, kind, split_k, C.byref(h)))
+        return cls(h)
+
+    def save(self, path: str):
+        _ck(lib().sptmm_weights_save(self.handle, os.fsencode(path)))
+
+    @classmethod
+    def load(cls, path: str) -> "Weights":
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_load(os.fsencode(path), C.byref(h)))
         return cls(h)
 
     def clone(self) -> "Weights":

@@ -2,6 +2,7 @@
 // memory / stream / event helpers.  See include/sptmm.h for the contract.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <new>
@@ -257,6 +258,130 @@ int sptmm_weights_info(const sptmm_weights *w, sptmm_winfo *out)
 }
 
 size_t sptmm_weights_bytes(const sptmm_weights *w) { return w ? w->bytes : 0; }
+
+// ---- weight files: a fixed little-endian header, then the device stream as it is ----
+namespace {
+struct FileHeader {
+    char magic[8];            // "SPTMMW1\0"
+    uint32_t header_bytes;    // sizeof(FileHeader)
+    uint32_t version;         // 1
+    int32_t kind, K, N, S, split_k, delta_bits, ragged;
+    int32_t half, L, G, W, n_lane, tasks;
+    int32_t task_stride, counts_bytes, n_min, n_max, index_shift;
+    uint64_t nnz, read_bytes, stream_bytes;
+    uint64_t fnv1a;           // of the header (this field zero) and the stream
+};
+static_assert(sizeof(FileHeader) == 8 + 4 + 4 + 7 * 4 + 6 * 4 + 5 * 4 + 4 * 8, "file header has no padding");
+const char FILE_MAGIC[8] = {'S', 'P', 'T', 'M', 'M', 'W', '1', 0};
+
+uint64_t fnv1a(const uint8_t *p, size_t n, uint64_t h = 1469598103934665603ull)
+{
+    for (size_t i = 0; i < n; ++i) h = (h ^ p[i]) * 1099511628211ull;
+    return h;
+}
+
+uint64_t file_checksum(FileHeader h, const std::vector<uint8_t> &stream)
+{
+    h.fnv1a = 0;
+    return fnv1a(stream.data(), stream.size(), fnv1a((const uint8_t *)&h, sizeof h));
+}
+}  // namespace
+
+int sptmm_weights_save(const sptmm_weights *w, const char *path)
+{
+    if (!w || !path) return fail(SPTMM_ERR_INVALID, "null pointer");
+    std::vector<uint8_t> host(w->bytes);
+    HIP_TRY(hipMemcpy(host.data(), w->dev, w->bytes, hipMemcpyDeviceToHost));
+    FileHeader h{};
+    memcpy(h.magic, FILE_MAGIC, 8);
+    h.header_bytes = (uint32_t)sizeof h;
+    h.version = 1;
+    const sptmm_winfo &i = w->info;
+    const Geometry &g = w->geo;
+    h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = i.ragged;
+    h.half = g.half, h.L = g.L, h.G = g.G, h.W = g.W, h.n_lane = g.n_lane, h.tasks = g.tasks;
+    h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max, h.index_shift = w->index_shift;
+    h.nnz = i.nnz, h.read_bytes = i.stream_bytes, h.stream_bytes = w->bytes;
+    h.fnv1a = file_checksum(h, host);
+    FILE *f = fopen(path, "wb");
+    if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s for writing", path);
+    const bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(host.data(), 1, host.size(), f) == host.size();
+    if (fclose(f) != 0 || !ok) return fail(SPTMM_ERR_INVALID, "short write to %s", path);
+    return SPTMM_OK;
+}
+
+int sptmm_weights_load(const char *path, sptmm_weights **out)
+{
+    if (!path || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
+    FILE *f = fopen(path, "rb");
+    if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s", path);
+    FileHeader h{};
+    std::vector<uint8_t> host;
+    int rc = SPTMM_OK;
+    if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || h.version != 1)
+        rc = fail(SPTMM_ERR_INVALID, "%s is not a weight file of this library", path);
+    // every field the kernels index with is checked against the stream size before anything is uploaded
+    if (!rc) {
+        Geometry g{};
+        size_t want = 0;
+        if (h.kind == SPTMM_KIND_I2S) {
+            want = sptmm_pack_i2s_bytes(h.K, h.N);
+        } else if (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA) {
+            const int max_split = h.kind == SPTMM_KIND_U16 ? 256 : 64;
+            const bool gaps = h.kind == SPTMM_KIND_DELTA;
+            if (gaps ? (h.delta_bits != 8 && h.delta_bits != 16) : h.delta_bits != 0) {
+                rc = fail(SPTMM_ERR_INVALID, "%s: bad gap width", path);
+            } else if (h.ragged) {
+                const int esz = gaps ? h.delta_bits / 8 : 2;
+                if (h.K <= 0 || h.N <= 0 || h.K % 16 || h.N % 16 || h.K + 64 > 65535 || make_ragged_geometry(h.N, h.split_k, max_split, &g) ||
+                    h.n_min < 1 || h.n_max < h.n_min || h.n_max > 65535 || h.counts_bytes != (int)ragged_counts_bytes(g.tasks) ||
+                    h.task_stride != (gaps ? 256 : 0) + 128 * esz * h.n_max ||
+                    h.index_shift != (gaps ? 0 : ragged_index_shift(h.K)))
+                    rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent ragged stream header", path);
+                else
+                    want = (size_t)h.counts_bytes + (size_t)h.task_stride * g.tasks;
+            } else {
+                if (check_shape(h.K, h.N, h.S) || make_geometry(h.N, h.S, h.split_k, max_split, &g) ||
+                    h.index_shift != (gaps ? 0 : u16_index_shift(h.K)))
+                    rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent stream header", path);
+                else
+                    want = gaps ? sptmm_pack_delta_bytes(h.N, h.S, h.split_k, h.delta_bits) : sptmm_pack_u16_bytes(h.N, h.S, h.split_k);
+            }
+            if (!rc && (g.half != h.half || g.L != h.L || g.G != h.G || g.W != h.W || g.n_lane != h.n_lane || g.tasks != h.tasks))
+                rc = fail(SPTMM_ERR_INVALID, "%s: geometry does not match the shape", path);
+        } else {
+            rc = fail(SPTMM_ERR_INVALID, "%s: unknown stream kind %d", path, h.kind);
+        }
+        if (!rc && (want == 0 || want != h.stream_bytes)) rc = fail(SPTMM_ERR_INVALID, "%s: stream size does not match the shape", path);
+    }
+    if (!rc) {
+        host.resize(h.stream_bytes);
+        if (fread(host.data(), 1, host.size(), f) != host.size() || fgetc(f) != EOF)
+            rc = fail(SPTMM_ERR_INVALID, "%s: truncated or oversized file", path);
+        else if (file_checksum(h, host) != h.fnv1a)
+            rc = fail(SPTMM_ERR_INVALID, "%s: checksum mismatch", path);
+    }
+    fclose(f);
+    if (rc) return rc;
+    if (h.ragged && (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA)) {
+        // the per-task counts are what the kernel trusts most: keep them inside [n_min, n_max]
+        const uint32_t *pre = (const uint32_t *)host.data();
+        const uint16_t *counts = (const uint16_t *)(host.data() + 16);
+        bool ok = pre[0] == RAGGED_MAGIC && pre[1] == (uint32_t)h.tasks && pre[2] == (uint32_t)h.n_max && pre[3] == (uint32_t)h.n_min;
+        for (int t = 0; ok && t < h.tasks; ++t) ok = counts[t] >= h.n_min && counts[t] <= h.n_max;
+        if (!ok) return fail(SPTMM_ERR_INVALID, "%s: corrupt count table", path);
+    }
+    sptmm_weights *w = new (std::nothrow) sptmm_weights();
+    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+    w->info = sptmm_winfo{h.kind, h.K, h.N, h.S, h.split_k, h.delta_bits, h.read_bytes, h.ragged, h.nnz};
+    w->geo = Geometry{h.N, h.half, h.split_k, h.L, h.G, h.W, h.n_lane, h.tasks};
+    w->task_stride = h.task_stride;
+    w->counts_bytes = h.counts_bytes;
+    w->n_min = h.n_min;
+    w->n_max = h.n_max;
+    w->index_shift = h.index_shift;
+    return finish_upload(w, host, out);
+}
 
 int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X, int M, int32_t *C, void *stream)
 {

@@ -1,0 +1,78 @@
+"""Weight files (sptmm_weights_save / _load): round trips on the GPU, refusals without one."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import oracle
+import sptmm_amd as sp
+
+
+def test_load_refuses_what_is_not_a_weight_file(tmp_path):
+    # these are rejected from the header alone, before any device call
+    p = tmp_path / "x.sptmm"
+    with pytest.raises(sp.SptmmError):
+        sp.Weights.load(str(p))  # missing
+    p.write_bytes(b"")
+    with pytest.raises(sp.SptmmError):
+        sp.Weights.load(str(p))
+    p.write_bytes(b"NOTSPTMM" + bytes(200))
+    with pytest.raises(sp.SptmmError):
+        sp.Weights.load(str(p))
+    hdr = bytearray(b"SPTMMW1\0" + (120).to_bytes(4, "little") + (1).to_bytes(4, "little") + bytes(104))
+    p.write_bytes(bytes(hdr))  # right magic, kind 0
+    with pytest.raises(sp.SptmmError) as e:
+        sp.Weights.load(str(p))
+    assert "kind" in str(e.value)
+
+
+@pytest.mark.gpu
+def test_save_load_round_trip_every_encoding(tmp_path):
+    sp.device_init(0)
+    K, N, S = 2560, 640, 1536
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    Wi = sp.generate_ternary_iid(K, N, 3, 0.3, 0.3)
+    X = oracle.make_x_i8(7, 4, K)
+    makers = {
+        "u16": lambda: sp.Weights.upload_u16(pos, neg, K, 32),
+        "u16_256": lambda: sp.Weights.upload_u16(pos, neg, K, 256),
+        "delta8": lambda: sp.Weights.upload_delta(pos, neg, K, 32),
+        "i2s": lambda: sp.Weights.upload_i2s(W),
+        "ragged_u16": lambda: sp.Weights.upload_dense(Wi, sp.KIND_U16, 32),
+        "ragged_delta": lambda: sp.Weights.upload_dense(Wi, sp.KIND_DELTA, 16),
+    }
+    for name, mk in makers.items():
+        print("weight file", name, flush=True)
+        sys.stdout.flush()
+        w = mk()
+        want = w.matmul(X)
+        path = str(tmp_path / (name + ".sptmm"))
+        w.save(path)
+        assert os.path.getsize(path) == 120 + w.nbytes
+        v = sp.Weights.load(path)
+        assert v.info == w.info and v.nbytes == w.nbytes
+        assert (v.matmul(X) == want).all()
+        assert (want == oracle.dense_i8(X, Wi if name.startswith("ragged") else W)).all()
+        w.free()
+        v.free()
+        # one flipped stream byte, a truncated file and trailing bytes are all refused
+        raw = bytearray(open(path, "rb").read())
+        raw[120 + len(raw) // 3] ^= 0x40
+        open(path, "wb").write(bytes(raw))
+        with pytest.raises(sp.SptmmError) as e:
+            sp.Weights.load(path)
+        assert "checksum" in str(e.value) or "corrupt" in str(e.value)
+        raw[120 + len(raw) // 3] ^= 0x40
+        open(path, "wb").write(bytes(raw[:-5]))
+        with pytest.raises(sp.SptmmError):
+            sp.Weights.load(path)
+        open(path, "wb").write(bytes(raw) + b"\0")
+        with pytest.raises(sp.SptmmError):
+            sp.Weights.load(path)
+        # a header that disagrees with the stream size
+        bad = bytearray(raw)
+        bad[20:24] = (K + 16).to_bytes(4, "little")  # K
+        open(path, "wb").write(bytes(bad))
+        with pytest.raises(sp.SptmmError):
+            sp.Weights.load(path)
