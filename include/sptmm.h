@@ -176,6 +176,16 @@ int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X_dev, int M, int32_t *C
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X_dev, int M, float *C_dev, void *stream);
 int sptmm_gemv_f32(const sptmm_weights *w, const float *X_dev, int M, float *C_dev, void *stream);
 
+/* The GEMV with its BitNet wrapper fused in: fp16 or bf16 activation rows are
+ * quantised to int8 while the tile is staged (per row s = 127 / max(|x|, 1e-5),
+ * q = clamp(rint(x*s), -127, 127), round-half-even), the sums run exactly as in
+ * sptmm_gemv_i8, and the output is Y[m][n] = (float)C[m][n] * (1/s_m) * w_scale
+ * in fp32 (evaluated in this order).  One launch where the unfused sequence takes
+ * three (quantise, GEMV, rescale).  The reference has the GEMV only; it passes
+ * an unused scale to its i2s kernel (main.cu:1862).  u16 and gap streams. */
+typedef enum sptmm_xtype { SPTMM_X_F16 = 1, SPTMM_X_BF16 = 2 } sptmm_xtype;
+int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *stream);
+
 /* `count` independent GEMVs of one shape in ONE launch: C[i] = X[i] . ws[i]
  * (int8 activations, u16 or gap streams that agree in K, N, S, split_k).  What a
  * decoder does with projections that share a shape; the reference launches its
@@ -204,7 +214,7 @@ int sptmm_event_elapsed_us(void *start, void *stop, double *us);
 /* The timing loop of measureKernel (main.cu:767-782) around `iters` GEMV
  * launches, kept native so that no interpreter sits between launches.  Launch i
  * uses ws[i % n_ws] (several device copies of one matrix defeat the last-level
- * cache).  act: 0 int8, 1 fp16, 2 fp32.  mode: 0 = back-to-back launches on one
+ * cache).  act: 0 int8, 1 fp16, 2 fp32, 3 / 4 sptmm_gemv_q8 on fp16 / bf16 rows.  mode: 0 = back-to-back launches on one
  * stream between two events; 1 = stream synchronize after every launch, as the
  * reference does (main.cu:1456); 2 = one rotation captured into a HIP graph and
  * replayed; 3 = every rotation is ONE sptmm_gemv_i8_batched launch of all n_ws

@@ -29,7 +29,7 @@ EXPORTS = [
     "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
-    "sptmm_gemv_f32", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
+    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel",
@@ -83,6 +83,7 @@ def lib() -> C.CDLL:
         L.sptmm_weights_load.argtypes = [C.c_char_p, C.POINTER(C.c_void_p)]
         for n in ("sptmm_gemv_i8", "sptmm_gemv_f16", "sptmm_gemv_f32"):
             getattr(L, n).argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.sptmm_gemv_q8.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p]
         L.sptmm_gemv_i8_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
         L.sptmm_free.argtypes = [C.c_void_p]
@@ -422,6 +423,26 @@ class Weights:
 
     def gemv_f32(self, X: DeviceBuffer, M: int, Cout: DeviceBuffer, stream: Stream | None = None):
         _ck(lib().sptmm_gemv_f32(self.handle, X.ptr, M, Cout.ptr, stream.handle if stream else None))
+
+    def gemv_q8(self, X: DeviceBuffer, x_type: int, M: int, w_scale: float, Yout: DeviceBuffer, stream: Stream | None = None):
+        """x_type 1 = fp16, 2 = bf16 (raw 16-bit patterns); Y = float32."""
+        _ck(lib().sptmm_gemv_q8(self.handle, X.ptr, x_type, M, w_scale, Yout.ptr, stream.handle if stream else None))
+
+    def matmul_q8(self, X: np.ndarray, w_scale: float = 1.0, bf16: bool = False) -> np.ndarray:
+        """Host convenience: X [M][K] float16 (or uint16 bf16 patterns with bf16=True) -> Y [M][N] float32."""
+        i = self.info
+        M, K = X.shape
+        assert K == i["K"] and X.dtype == (np.uint16 if bf16 else np.float16)
+        xb = DeviceBuffer.from_numpy(X)
+        yb = DeviceBuffer(4 * M * i["N"])
+        yb.fill(0xFF)
+        try:
+            self.gemv_q8(xb, 2 if bf16 else 1, M, w_scale, yb)
+            device_sync()
+            return yb.to_numpy(np.float32, (M, i["N"]))
+        finally:
+            xb.free()
+            yb.free()
 
     def matmul(self, X: np.ndarray) -> np.ndarray:
         """Host convenience: upload X [M][K], run on the device, download C [M][N]."""

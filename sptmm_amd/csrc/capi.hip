@@ -87,7 +87,8 @@ int finish_upload(sptmm_weights *w, const std::vector<uint8_t> &host, sptmm_weig
 }
 
 int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *stream, ActType act, int batch = 0,
-                const void *const *bw = nullptr, const void *const *bx = nullptr, void *const *bc = nullptr)
+                const void *const *bw = nullptr, const void *const *bx = nullptr, void *const *bc = nullptr, int quant = 0,
+                float w_scale = 1.f)
 {
     if (!w || !X || !C) return fail(SPTMM_ERR_INVALID, "null pointer");
     if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
@@ -114,6 +115,8 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.ragged = w->info.ragged;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
+    a.quant = quant;
+    a.w_scale = w_scale;
     a.batch = batch;
     a.batch_w = bw;
     a.batch_X = bx;
@@ -410,6 +413,13 @@ int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X
     return gemv_common(ws[0], X[0], M, C[0], stream, ACT_I8, count, wp.data(), xp.data(), cp.data());
 }
 
+int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X, int x_type, int M, float w_scale, float *Y, void *stream)
+{
+    if (x_type != SPTMM_X_F16 && x_type != SPTMM_X_BF16) return fail(SPTMM_ERR_INVALID, "x_type must be SPTMM_X_F16 or SPTMM_X_BF16");
+    if (w && w->info.kind == SPTMM_KIND_I2S) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes u16 or gap streams");
+    return gemv_common(w, X, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, x_type, w_scale);
+}
+
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X, int M, float *C, void *stream)
 {
     return gemv_common(w, X, M, C, stream, ACT_F16);
@@ -504,8 +514,13 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
                        int mode, void *stream, double *us_per_call)
 {
     if (!ws || n_ws < 1 || !X || !C || iters < 1 || !us_per_call) return fail(SPTMM_ERR_INVALID, "bad argument");
-    if (act < ACT_I8 || act > ACT_F32 || mode < 0 || mode > 3) return fail(SPTMM_ERR_INVALID, "bad act or mode");
+    if (act < 0 || act > 4 || mode < 0 || mode > 3) return fail(SPTMM_ERR_INVALID, "bad act or mode");
     if (mode == 3 && act != ACT_I8) return fail(SPTMM_ERR_UNSUPPORTED, "batched timing takes int8 activations");
+    // act 3 / 4: the quantising GEMV on fp16 / bf16 rows (w_scale 1)
+    auto launch = [&](const sptmm_weights *w) {
+        return act >= 3 ? sptmm_gemv_q8(w, (const uint16_t *)X, act == 3 ? SPTMM_X_F16 : SPTMM_X_BF16, M, 1.0f, (float *)C, stream)
+                        : gemv_common(w, X, M, C, stream, (ActType)act);
+    };
     if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_measure_gemv needs a stream made by sptmm_stream_create");
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -527,7 +542,7 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
     if (mode == 2) {
         // one rotation over the weight copies becomes one graph; replay it iters/n_ws times
         M_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-        for (int i = 0; i < n_ws && rc == SPTMM_OK; ++i) rc = gemv_common(ws[i], X, M, C, st, (ActType)act);
+        for (int i = 0; i < n_ws && rc == SPTMM_OK; ++i) rc = launch(ws[i]);
         hipError_t ce = hipStreamEndCapture(st, &graph);
         if (rc != SPTMM_OK) goto done;
         M_TRY(ce);
@@ -559,7 +574,7 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
     } else {
         M_TRY(hipEventRecord(e0, st));
         for (int i = 0; i < iters; ++i) {
-            rc = gemv_common(ws[i % n_ws], X, M, C, st, (ActType)act);
+            rc = launch(ws[i % n_ws]);
             if (rc != SPTMM_OK) goto done;
             if (mode == 1) M_TRY(hipStreamSynchronize(st));
         }

@@ -101,6 +101,8 @@ struct GemvArgs {
     int n_min, n_max;   // smallest / largest per-task entry count
     int compute_units;
     int lds_limit;
+    int quant = 0;        // 1 / 2: X holds fp16 / bf16 rows, quantised to int8 in the kernel; C receives floats
+    float w_scale = 1.f;  // quantising launches: factor applied to every output
     // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each
     int batch = 0;
     const void *const *batch_w = nullptr;

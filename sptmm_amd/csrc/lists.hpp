@@ -314,6 +314,8 @@ struct ListParams {
     int task_stride;             // ragged streams: bytes between tasks
     int counts_bytes;            // ragged streams: bytes of the count table (with its preamble) in front of the tasks
     int iters;  // tasks each wavefront walks: ceil(tasks / (gridDim.x * waves))
+    int quant;      // quantising kernels: X holds 1 = fp16, 2 = bf16 values
+    float w_scale;  // quantising kernels: factor applied to every output
 };
 
 constexpr int LISTS_MAX_WAVES = 8;  // 512 threads: two wavefronts per SIMD, 256 VGPRs each
@@ -342,7 +344,70 @@ __device__ __forceinline__ Round load_round(const uint4 *wp, int r)
     return x;
 }
 
-template <typename Act, int MT, int MODE, bool PRE, bool VAR>
+// Activation quantisation in front of the integer GEMV (per row: s = 127 / max(|x|, 1e-5),
+// q = clamp(rint(x * s), -127, 127)) for the kernels that take fp16 / bf16 rows and
+// hand back floats.  Item = 16 consecutive k of all MT rows, as in Stager.
+template <int MT> struct Quantiser {
+    static constexpr int HOLD = MT == 1 ? 2 : 0;  // items a thread keeps in registers between the two passes (the rest is read twice)
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+    // 2 x 16 bytes per row: the item's 16 values of row m0 + m (rows past M read as zero)
+    static __device__ __forceinline__ void load(const unsigned short *X, int M, int K, int m0, int item, uint4 (&r)[2 * MT])
+    {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                r[2 * m + j] = (m0 + m < M) ? reinterpret_cast<const uint4 *>(X + (size_t)(m0 + m) * K)[(size_t)item * 2 + j]
+                                            : make_uint4(0, 0, 0, 0);
+    }
+    // Running maxima of |x| as bit patterns, two per register: for fp16 and bf16 alike, clearing
+    // the sign bit leaves patterns that order like the magnitudes they encode.
+    static __device__ __forceinline__ void absmax(const uint4 (&r)[2 * MT], u32 (&mx)[MT])
+    {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const u32 d = comp(r[2 * m + c / 4], c % 4) & 0x7fff7fffu;
+                mx[m] = __builtin_bit_cast(u32, __builtin_elementwise_max(__builtin_bit_cast(u16x2, mx[m]), __builtin_bit_cast(u16x2, d)));
+            }
+    }
+    static __device__ __forceinline__ float magnitude(u32 packed, int kind)
+    {
+        const u32 bits = (packed >> 16) > (packed & 0xffffu) ? packed >> 16 : packed & 0xffffu;
+        return kind == 2 ? __builtin_bit_cast(float, bits << 16) : (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
+    }
+    template <int KIND> static __device__ __forceinline__ float value(u32 d, int hi)
+    {
+        if constexpr (KIND == 2) return __builtin_bit_cast(float, hi ? d & 0xffff0000u : d << 16);
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)(hi ? d >> 16 : d & 0xffffu));
+    }
+    // -> the 16 int8 of every row, packed as the int8 kernels' own activation loads would deliver them.
+    // No clamp: |x| <= a and s = 127 / a keep |x * s| below 127.5.
+    template <int KIND> static __device__ __forceinline__ void quantise_as(const uint4 (&r)[2 * MT], const float (&s)[MT], uint4 (&q)[MT])
+    {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            u32 w[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int v = (int)__builtin_rintf(value<KIND>(comp(r[2 * m + e / 8], (e / 2) % 4), e & 1) * s[m]);
+                w[e / 4] |= ((u32)v & 0xffu) << (8 * (e % 4));
+            }
+            q[m] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+    static __device__ __forceinline__ void quantise(const uint4 (&r)[2 * MT], int kind, const float (&s)[MT], uint4 (&q)[MT])
+    {
+        if (kind == 2)
+            quantise_as<2>(r, s, q);
+        else
+            quantise_as<1>(r, s, q);
+    }
+};
+
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, bool QUANT = false>
 struct ListsBody {
     typedef typename Acc<Act>::type A;
     typedef Stager<Act, MT> St;
@@ -390,15 +455,28 @@ struct ListsBody {
         int task = blockIdx.x * waves + wave;
         const int task_step = gridDim.x * waves;
         const Act *X = reinterpret_cast<const Act *>(p.X);
+        typedef Quantiser<MT> Q;
+        const unsigned short *Xq = reinterpret_cast<const unsigned short *>(p.X);
+        // quantising kernels: behind the per-wavefront sums, one row maximum per wavefront and the rows' 1/s
+        float *qmax = reinterpret_cast<float *>(part + LISTS_MAX_WAVES * MT), *qinv = qmax + LISTS_MAX_WAVES * MT;
 
         // 1. every wavefront's activation loads enter the memory pipeline ahead of
         //    any stream load of the workgroup ...
         const int items = p.K / 16;
-        uint4 xr[St::XI][St::NLOAD];
+        uint4 xr[QUANT ? 1 : St::XI][St::NLOAD];
+        uint4 xq[QUANT && Q::HOLD > 0 ? Q::HOLD : 1][2 * MT];
+        if constexpr (QUANT) {
 #pragma unroll
-        for (int i = 0; i < St::XI; ++i) {
-            const int item = tid + i * nt;
-            St::load(X, p.M, p.K, m0, item < items ? item : items - 1, xr[i]);
+            for (int i = 0; i < Q::HOLD; ++i) {
+                const int item = tid + i * nt;
+                Q::load(Xq, p.M, p.K, m0, item < items ? item : items - 1, xq[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < St::XI; ++i) {
+                const int item = tid + i * nt;
+                St::load(X, p.M, p.K, m0, item < items ? item : items - 1, xr[i]);
+            }
         }
         // ragged: the first task's entry count travels with the activation loads, so it is there
         // long before the tile is; every later count is asked for one task ahead
@@ -419,9 +497,52 @@ struct ListsBody {
         }
 
         // 3. ... and the tile is written while the stream is still in flight.
+        if constexpr (QUANT) {
+            // row maxima: own items (held, and beyond them re-read later), wavefront, workgroup
+            u32 mb[MT];
 #pragma unroll
-        for (int i = 0; i < St::XI; ++i)
-            if (tid + i * nt < items) St::store(smem, tid + i * nt, xr[i]);
+            for (int m = 0; m < MT; ++m) mb[m] = 0u;
+#pragma unroll
+            for (int i = 0; i < Q::HOLD; ++i) Q::absmax(xq[i], mb);  // (a clamped duplicate changes no maximum)
+            for (int item = tid + Q::HOLD * nt; item < items; item += nt) {
+                uint4 r[2 * MT];
+                Q::load(Xq, p.M, p.K, m0, item, r);
+                Q::absmax(r, mb);
+            }
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                float mx = Q::magnitude(mb[m], p.quant);
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                if (lane == 0) qmax[wave * MT + m] = mx;
+            }
+            __syncthreads();
+            float sc[MT];
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                float a = 0.f;
+                for (int w = 0; w < waves; ++w) a = fmaxf(a, qmax[w * MT + m]);
+                a = fmaxf(a, 1e-5f);
+                sc[m] = 127.0f / a;
+                if (tid == 0) qinv[m] = a / 127.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < Q::HOLD; ++i)
+                if (tid + i * nt < items) {
+                    Q::quantise(xq[i], p.quant, sc, xr[0]);
+                    St::store(smem, tid + i * nt, xr[0]);
+                }
+            for (int item = tid + Q::HOLD * nt; item < items; item += nt) {
+                uint4 r[2 * MT];
+                Q::load(Xq, p.M, p.K, m0, item, r);
+                Q::quantise(r, p.quant, sc, xr[0]);
+                St::store(smem, item, xr[0]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < St::XI; ++i)
+                if (tid + i * nt < items) St::store(smem, tid + i * nt, xr[i]);
+        }
         if constexpr (RF > EARLY) {
             const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
 #pragma unroll
@@ -433,10 +554,12 @@ struct ListsBody {
                 for (int i = EARLY; i < RING; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
             }
         }
-        for (int item = tid + St::XI * nt; item < items; item += nt) {
-            uint4 r[St::NLOAD];
-            St::load(X, p.M, p.K, m0, item, r);
-            St::store(smem, item, r);
+        if constexpr (!QUANT) {
+            for (int item = tid + St::XI * nt; item < items; item += nt) {
+                uint4 r[St::NLOAD];
+                St::load(X, p.M, p.K, m0, item, r);
+                St::store(smem, item, r);
+            }
         }
         // rows K.. read as zero (biased bytes: 128)
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
@@ -444,6 +567,10 @@ struct ListsBody {
         __syncthreads();
 
         A *C = reinterpret_cast<A *>(p.C);
+        float *Cf = reinterpret_cast<float *>(p.C);  // quantising kernels: acc / s * w_scale
+        float back[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) back[m] = QUANT ? qinv[m] : 0.f;
         const int L = 1 << p.logL;
         for (int it = 0; it < p.iters; ++it, task += task_step) {
             const bool active = task < p.tasks;
@@ -581,7 +708,12 @@ struct ListsBody {
                     const int col = (task << (6 - p.logL)) + (lane >> p.logL);
 #pragma unroll
                     for (int m = 0; m < MT; ++m)
-                        if (m0 + m < p.M) C[(size_t)(m0 + m) * p.N + col] = acc.acc[m];
+                        if (m0 + m < p.M) {
+                            if constexpr (QUANT)
+                                Cf[(size_t)(m0 + m) * p.N + col] = (float)acc.acc[m] * back[m] * p.w_scale;
+                            else
+                                C[(size_t)(m0 + m) * p.N + col] = acc.acc[m];
+                        }
                 }
             } else {
                 // second pass: the W wavefronts of a column meet in a small LDS buffer
@@ -596,7 +728,12 @@ struct ListsBody {
                     for (int m = 0; m < MT; ++m) {
                         A s = (A)0;
                         for (int w = 0; w < p.W; ++w) s += part[(wave + w) * MT + m];
-                        if (m0 + m < p.M) C[(size_t)(m0 + m) * p.N + col] = s;
+                        if (m0 + m < p.M) {
+                            if constexpr (QUANT)
+                                Cf[(size_t)(m0 + m) * p.N + col] = (float)s * back[m] * p.w_scale;
+                            else
+                                C[(size_t)(m0 + m) * p.N + col] = s;
+                        }
                     }
                 }
                 __syncthreads();
@@ -611,11 +748,11 @@ struct ListsBody {
 // wavefronts then walk tasks blockIdx.x*waves + wave, + gridDim.x*waves, ...
 // blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
 // exactly RF full rounds (straight-line body); RF == 0: any length (ring).
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool QUANT = false>
 __global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    ListsBody<Act, MT, MODE, PRE, VAR>::template run<RF>(p, smem);
+    ListsBody<Act, MT, MODE, PRE, VAR, QUANT>::template run<RF>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -707,7 +844,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     const int grid_x = blocks < slots ? blocks : slots;
     const int iters = (blocks + grid_x - 1) / grid_x;
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
-                 a.task_stride, a.counts_bytes, iters};
+                 a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale};
     size_t lds = (size_t)(a.K + 64) * SLOT + (size_t)wpb * MT * sizeof(typename Acc<Act>::type);
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
@@ -732,6 +869,21 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             return SPTMM_OK;
         } else {
             return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take int8 activations");
+        }
+    }
+    if (a.quant) {
+        if constexpr (sizeof(Act) == 1) {
+            auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, true>;
+            // + room for the per-wavefront sums of a full workgroup, the row maxima and the rows' 1/s
+            lds = (size_t)(a.K + 64) * SLOT + (size_t)(2 * LISTS_MAX_WAVES + 1) * MT * 4;
+            if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
+            static std::atomic<size_t> lds_granted_q{48 * 1024};
+            if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_q)) return rc;
+            hipLaunchKernelGGL(kern, grid, block, lds, st, p);
+            hipError_t e = hipGetLastError();
+            return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel (quantising) launch");
+        } else {
+            return fail(SPTMM_ERR_INVALID, "quantising launches go through the int8 kernels");
         }
     }
     auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF>;

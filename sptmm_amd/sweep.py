@@ -5,6 +5,7 @@
     python -m sptmm_amd.sweep headline  # K=6912 N=2560 S=4096, M in {1, 4}
     python -m sptmm_amd.sweep fused     # the layer with q+k+v (N=3840) and gate+up (N=13824) as single launches,
                                         # the fusions the reference benchmarks (main.cu:1107-1190): 4 launches per layer
+    python -m sptmm_amd.sweep q8        # sptmm_gemv_q8 (fp16 rows quantised in the kernel, float output) against sptmm_gemv_i8
     python -m sptmm_amd.sweep ragged    # the same four launches on matrices with independent entries (30 % +1, 30 % -1):
                                         # columns differ in nonzeros, streams carry per-task counts
 
@@ -131,6 +132,35 @@ def layer_sequence(shapes, M, st, rows, iid=None):
     cb.free()
 
 
+def q8_rows(st, rows):
+    """The fused quantise -> GEMV -> rescale launch against the plain int8 GEMV, same streams."""
+    for name, K, N, S, split in (("headline", 6912, 2560, 4096, 32), ("qkv", 2560, 3840, 1536, 32), ("gate+up", 2560, 13824, 1536, 16),
+                                 ("down", 6912, 2560, 4160, 32)):
+        _, pos, neg = sp.generate_ternary(K, N, S)
+        for M in (1, 4):
+            rng = np.random.default_rng(M)
+            xh = sp.DeviceBuffer.from_numpy(rng.standard_normal((M, K)).astype(np.float16))
+            xi = sp.DeviceBuffer.from_numpy(sp.make_x_i8(M, M, K))
+            cb = sp.DeviceBuffer(4 * M * N)
+            for enc in ("u16", "delta"):
+                w = sp.Weights.upload_u16(pos, neg, K, split) if enc == "u16" else sp.Weights.upload_delta(pos, neg, K, split)
+                n = copies_for(w.nbytes)
+                cps = [w] + [w.clone() for _ in range(n - 1)]
+                out = {"shape": name, "K": K, "N": N, "M": M, "enc": "%s/%d" % (enc, split)}
+                for act, xb, tag in ((0, xi, "i8"), (3, xh, "q8")):
+                    sp.measure_gemv(cps[:1], act, xb, M, cb, 200, 0, st)
+                    out[tag + "_warm_us"] = round(min(sp.measure_gemv(cps[:1], act, xb, M, cb, 2000, 0, st) for _ in range(3)), 3)
+                    sp.measure_gemv(cps, act, xb, M, cb, 2 * n, 0, st)
+                    out[tag + "_cold_us"] = round(min(sp.measure_gemv(cps, act, xb, M, cb, 2000, 0, st) for _ in range(3)), 3)
+                print("%-8s M=%d %-8s int8 GEMV warm %6.2f cold %6.2f us | fused q8 warm %6.2f cold %6.2f us"
+                      % (name, M, out["enc"], out["i8_warm_us"], out["i8_cold_us"], out["q8_warm_us"], out["q8_cold_us"]), flush=True)
+                rows.append(out)
+                for c in cps:
+                    c.free()
+            for b in (xh, xi, cb):
+                b.free()
+
+
 def main(argv):
     which = argv[1] if len(argv) > 1 else "layer"
     info = sp.device_init(0)
@@ -154,12 +184,14 @@ def main(argv):
         if which != "layer":
             for M in (1, 4):
                 layer_sequence(shapes, M, st, rows, iid=(0.3, 0.3) if which == "ragged" else None)
+    elif which == "q8":
+        q8_rows(st, rows)
     elif which == "large":
         run_shape("large", 13824, 5120, 8320, (1, 8, 16), (32, 64), st, rows)
     elif which == "headline":
         run_shape("headline", 6912, 2560, 4096, (1, 4), (16, 32, 64), st, rows)
     else:
-        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged")
+        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged|q8")
     assert all(r.get("ok", True) for r in rows), "encodings disagree"
     print(json.dumps({"device": info["arch"], "rows": rows}))
 
