@@ -187,7 +187,7 @@ typedef enum sptmm_xtype { SPTMM_X_F16 = 1, SPTMM_X_BF16 = 2 } sptmm_xtype;
 int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *stream);
 
 /* `count` independent GEMVs of one shape in ONE launch: C[i] = X[i] . ws[i]
- * (int8 activations, u16 or gap streams that agree in K, N, S, split_k).  What a
+ * (int8 activations; streams of one kind that agree in K, N, S, split_k).  What a
  * decoder does with projections that share a shape; the reference launches its
  * kernels one at a time (main.cu:994-1459), so every launch there pays the
  * dispatch latency that this call pays once.  The pointer arrays are host

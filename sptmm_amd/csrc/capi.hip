@@ -401,7 +401,6 @@ int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X
     for (int i = 0; i < count; ++i) {
         if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
         const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
-        if (b.kind == SPTMM_KIND_I2S) return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take u16 or gap streams");
         if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
             a.ragged != b.ragged || ws[0]->task_stride != ws[i]->task_stride ||
             ws[0]->n_min != ws[i]->n_min)

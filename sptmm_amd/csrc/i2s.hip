@@ -38,9 +38,8 @@ struct I2sParams {
 // Codes 1..3 are used as they are in dot4; the "-2" of the decode
 // (bitnet_kernels.cuh:70) becomes one subtraction of 2*sum(X row) at the end.
 template <int MT>
-__global__ void __launch_bounds__(1024) i2s_kernel(I2sParams p)
+__device__ __forceinline__ void i2s_body(const I2sParams &p, unsigned char *smem)
 {
-    extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lx = reinterpret_cast<int8_t *>(smem);                       // [MT][Kp]
     int *part = reinterpret_cast<int *>(smem + (size_t)MT * p.Kp);      // [waves][16][MT]
     int *sums = part + (blockDim.x >> 6) * 16 * MT;                      // [waves][MT]
@@ -128,6 +127,31 @@ __global__ void __launch_bounds__(1024) i2s_kernel(I2sParams p)
     }
 }
 
+template <int MT>
+__global__ void __launch_bounds__(1024) i2s_kernel(I2sParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    i2s_body<MT>(p, smem);
+}
+
+// Several independent GEMVs of one shape in one launch: blockIdx.z picks the (stream, X, C) triple.
+constexpr int I2S_BATCH_MAX = 32;
+struct I2sBatch {
+    const uint4 *w[I2S_BATCH_MAX];
+    const int8_t *X[I2S_BATCH_MAX];
+    int *C[I2S_BATCH_MAX];
+};
+
+template <int MT>
+__global__ void __launch_bounds__(1024) i2s_kernel_batched(I2sParams p, I2sBatch b)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    p.w = b.w[blockIdx.z];
+    p.X = b.X[blockIdx.z];
+    p.C = b.C[blockIdx.z];
+    i2s_body<MT>(p, smem);
+}
+
 __global__ void __launch_bounds__(256) copy_kernel(uint4 *dst, const uint4 *src, size_t n16)
 {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
@@ -155,10 +179,29 @@ static int launch_i2s_t(const GemvArgs &a, hipStream_t st, int waves)
     const int Kp = i2s_padded_k(a.K);
     I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256};
     size_t lds = (size_t)MT * Kp + (size_t)waves * 16 * MT * 4 + (size_t)waves * MT * 4;
+    dim3 grid(a.N / 16, (a.M + MT - 1) / MT), block(64 * waves);
+    if (a.batch) {
+        auto kern = i2s_kernel_batched<MT>;
+        static std::atomic<size_t> lds_granted_b{48 * 1024};
+        if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_b)) return rc;
+        for (int first = 0; first < a.batch; first += I2S_BATCH_MAX) {
+            I2sBatch b{};
+            const int n = a.batch - first < I2S_BATCH_MAX ? a.batch - first : I2S_BATCH_MAX;
+            for (int i = 0; i < n; ++i) {
+                b.w[i] = (const uint4 *)a.batch_w[first + i];
+                b.X[i] = (const int8_t *)a.batch_X[first + i];
+                b.C[i] = (int *)a.batch_C[first + i];
+            }
+            grid.z = n;
+            hipLaunchKernelGGL(kern, grid, block, lds, st, p, b);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return hip_fail(e, "i2s_kernel_batched launch");
+        }
+        return SPTMM_OK;
+    }
     auto kern = i2s_kernel<MT>;
     static std::atomic<size_t> lds_granted{48 * 1024};
     if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
-    dim3 grid(a.N / 16, (a.M + MT - 1) / MT), block(64 * waves);
     hipLaunchKernelGGL(kern, grid, block, lds, st, p);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "i2s_kernel launch");

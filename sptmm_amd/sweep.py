@@ -5,6 +5,7 @@
     python -m sptmm_amd.sweep headline  # K=6912 N=2560 S=4096, M in {1, 4}
     python -m sptmm_amd.sweep fused     # the layer with q+k+v (N=3840) and gate+up (N=13824) as single launches,
                                         # the fusions the reference benchmarks (main.cu:1107-1190): 4 launches per layer
+    python -m sptmm_amd.sweep density   # K=6912 N=2560 M=1 at S = 256 ... 4096: where the index lists move fewer bytes than 2 bits per weight
     python -m sptmm_amd.sweep q8        # sptmm_gemv_q8 (fp16 rows quantised in the kernel, float output) against sptmm_gemv_i8
     python -m sptmm_amd.sweep ragged    # the same four launches on matrices with independent entries (30 % +1, 30 % -1):
                                         # columns differ in nonzeros, streams carry per-task counts
@@ -78,7 +79,7 @@ def run_shape(name, K, N, S, Ms, splits, st, rows, iid=None):
                 ref = got
             ok = bool((got == ref).all())
             nbytes = w.info["stream_bytes"] + M * K + 4 * M * N  # what one GEMV reads and writes
-            warm, cold, bat = time_weights(w, X, M, N, st, enc != "i2s")
+            warm, cold, bat = time_weights(w, X, M, N, st, True)
             w.free()
             rows.append({"shape": name, "K": K, "N": N, "S": S, "M": M, "enc": enc, "bytes": nbytes, "ok": ok,
                          "warm_us": round(warm, 3), "cold_us": round(cold, 3),
@@ -184,6 +185,9 @@ def main(argv):
         if which != "layer":
             for M in (1, 4):
                 layer_sequence(shapes, M, st, rows, iid=(0.3, 0.3) if which == "ragged" else None)
+    elif which == "density":
+        for S in (256, 512, 1024, 2048, 4096):
+            run_shape("S=%d" % S, 6912, 2560, S, (1,), (32,), st, rows)
     elif which == "q8":
         q8_rows(st, rows)
     elif which == "large":
@@ -191,7 +195,7 @@ def main(argv):
     elif which == "headline":
         run_shape("headline", 6912, 2560, 4096, (1, 4), (16, 32, 64), st, rows)
     else:
-        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged|q8")
+        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged|density|q8")
     assert all(r.get("ok", True) for r in rows), "encodings disagree"
     print(json.dumps({"device": info["arch"], "rows": rows}))
 

@@ -353,13 +353,13 @@ def test_streams_and_clone():
 
 
 # ------------------------------------------------------------------ batched launch
-@pytest.mark.parametrize("kind", ["u16", "delta"])
+@pytest.mark.parametrize("kind", ["u16", "delta", "i2s"])
 @pytest.mark.parametrize("M,count", [(1, 3), (4, 5), (1, 40)])
 def test_batched_launch_equals_single_launches(kind, M, count):
     K, N, S = 2560, 640, 1536
-    _, pos, neg = matrix(K, N, S)
-    up = sp.Weights.upload_u16 if kind == "u16" else sp.Weights.upload_delta
-    base = up(pos, neg, K, 32)
+    W, pos, neg = matrix(K, N, S, dense=True)
+    base = (sp.Weights.upload_i2s(W) if kind == "i2s" else sp.Weights.upload_u16(pos, neg, K, 32) if kind == "u16"
+            else sp.Weights.upload_delta(pos, neg, K, 32))
     ws = [base] + [base.clone() for _ in range(count - 1)]
     Xs = [x_i8(9000 + i, M, K) for i in range(count)]
     xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
