@@ -71,10 +71,11 @@ def main():
     ap.add_argument("--steps", type=int, default=256, help="timed steps; one step = one launch of BATCH GEMVs")
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="single,others",
+    ap.add_argument("--legs", default="single,others,ceiling",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, "
                          "sync-each-call), others (delta and i2s encodings), copy (4 launches of a 1 GiB copy kernel, for counter "
-                         "calibration); profiling runs use --legs none or --legs copy")
+                         "calibration), ceiling (a pure streaming read of as many bytes as one step moves: the practical HBM read "
+                         "ceiling on this box); profiling runs use --legs none or --legs copy")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported "
@@ -145,6 +146,16 @@ def main():
         src.free()
         dst.free()
 
+    ceiling = None
+    if "ceiling" in legs:
+        # the same bytes as one headline step, read with the kernels' own load instruction and thrown away
+        nb = nbytes * BATCH // 16 * 16
+        buf = sp.DeviceBuffer(nb)
+        buf.fill(1)
+        best = min(sp.read_kernel(buf, nb, st, 20, wgs) for wgs in (256, 512, 4096) for _ in range(2))
+        buf.free()
+        ceiling = {"bytes": nb, "us": round(best, 2), "gbps": round(nb / best / 1e3, 1)}
+
     others = {}
     if "others" in legs:
         for name, mk in (("delta8_split32", lambda: sp.Weights.upload_delta(pos, neg, K, SPLIT)),
@@ -191,6 +202,10 @@ def main():
                      "kernel": "lists_kernel_batched<int8, MT=1, u16>", "launch_us": round(launch_us, 2),
                      "algorithmic_bytes_per_launch": nbytes * BATCH},
     }
+    if ceiling:
+        # not the roofline's peak (that stays the published 8 TB/s): what a pure read of the same size reaches here
+        out["roofline"]["streaming_read_ceiling"] = ceiling
+        out["roofline"]["frac_of_streaming_read"] = round(gbps / ceiling["gbps"], 4)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline((pos, neg))
     w.free()

@@ -10,7 +10,7 @@ __all__ = [
     "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
     "generate_ternary_iid", "dense_from_i2s_words",
-    "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel",
+    "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
     "device_sync", "measure_gemv", "gemv_i8_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
 
@@ -32,7 +32,7 @@ EXPORTS = [
     "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
-    "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel",
+    "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
 ]
 
 
@@ -93,6 +93,7 @@ def lib() -> C.CDLL:
         L.sptmm_measure_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                          C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         L.sptmm_copy_kernel.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.sptmm_read_kernel.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         L.sptmm_make_x_i8.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p]
         L.sptmm_generate_ternary_iid.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_double, C.c_double, C.c_void_p]
         for n in ("sptmm_stream_create", "sptmm_event_create"):
@@ -349,6 +350,17 @@ def gemv_i8_batched(weights, Xs, Cs, M: int, stream: "Stream | None" = None):
 
 def device_sync():
     _ck(lib().sptmm_device_sync())
+
+
+def read_kernel(src: DeviceBuffer, nbytes: int, stream: Stream, launches: int = 20, workgroups: int = 0) -> float:
+    """Mean microseconds per launch of a pure streaming read of `nbytes` of `src`."""
+    sink = DeviceBuffer(16)
+    us = C.c_double()
+    try:
+        _ck(lib().sptmm_read_kernel(src.ptr, nbytes, sink.ptr, workgroups, launches, stream.handle, C.byref(us)))
+    finally:
+        sink.free()
+    return us.value
 
 
 def copy_kernel(dst: DeviceBuffer, src: DeviceBuffer, nbytes: int, stream: Stream | None = None):

@@ -592,6 +592,29 @@ done:
     return rc;
 }
 
+int sptmm_read_kernel(const void *src, size_t bytes, void *sink, int workgroups, int launches, void *stream, double *us_per_launch)
+{
+    if (!src || !sink || launches < 1 || !us_per_launch) return fail(SPTMM_ERR_INVALID, "bad argument");
+    if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_read_kernel needs a stream made by sptmm_stream_create");
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0));
+    HIP_TRY(hipEventCreate(&e1));
+    int rc = launch_read(src, bytes, sink, workgroups, stream);  // untimed first launch
+    hipError_t e = hipEventRecord(e0, st);
+    for (int i = 0; i < launches && rc == SPTMM_OK; ++i) rc = launch_read(src, bytes, sink, workgroups, stream);
+    if (e == hipSuccess) e = hipEventRecord(e1, st);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != SPTMM_OK) return rc;
+    if (e != hipSuccess) return hip_fail(e, "timing the read kernel");
+    *us_per_launch = (double)ms * 1000.0 / launches;
+    return SPTMM_OK;
+}
+
 int sptmm_copy_kernel(void *dst, const void *src, size_t bytes, void *stream)
 {
     if (!dst || !src) return fail(SPTMM_ERR_INVALID, "null pointer");

@@ -123,5 +123,6 @@ int launch_ragged_runs16(const GemvArgs &a, ActType act, void *stream);      // 
 int launch_delta(const GemvArgs &a, ActType act, void *stream);
 int launch_i2s(const GemvArgs &a, void *stream);
 int launch_copy(void *dst, const void *src, size_t bytes, void *stream);
+int launch_read(const void *src, size_t bytes, void *sink, int workgroups, void *stream);
 
 }  // namespace sptmm
