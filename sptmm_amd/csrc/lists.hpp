@@ -894,13 +894,13 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel launch");
 }
 
-// Straight-line bodies exist for the int8 paths of the u16 and 8-bit run streams
+// Straight-line bodies exist for the u16 and 8-bit run streams
 // with 1, 2, 3, 4, 6 or 8 full rounds per task (ragged streams: for the shortest
 // task, when the longest has at most XMAX more); everything else takes the ring.
 template <typename Act, int MT, int MODE, bool PRE, bool VAR>
 static int launch_lists_t(const GemvArgs &a, hipStream_t st)
 {
-    if constexpr (sizeof(Act) == 1 && MODE < 2) {
+    if constexpr (MODE < 2) {
         constexpr int E16 = MODE == 1 ? 16 : 8;
         int rf = (VAR ? a.n_min : a.n_lane) / E16;
         if constexpr (VAR) {

@@ -6,6 +6,7 @@
     python -m sptmm_amd.sweep fused     # the layer with q+k+v (N=3840) and gate+up (N=13824) as single launches,
                                         # the fusions the reference benchmarks (main.cu:1107-1190): 4 launches per layer
     python -m sptmm_amd.sweep density   # K=6912 N=2560 M=1 at S = 256 ... 4096: where the index lists move fewer bytes than 2 bits per weight
+    python -m sptmm_amd.sweep float     # fp16 / fp32 activations (the gap stream with fp16 rows is the benchmark's third configuration)
     python -m sptmm_amd.sweep q8        # sptmm_gemv_q8 (fp16 rows quantised in the kernel, float output) against sptmm_gemv_i8
     python -m sptmm_amd.sweep ragged    # the same four launches on matrices with independent entries (30 % +1, 30 % -1):
                                         # columns differ in nonzeros, streams carry per-task counts
@@ -162,6 +163,34 @@ def q8_rows(st, rows):
                 b.free()
 
 
+def float_rows(st, rows):
+    """fp16 / fp32 activations (fp32 sums) against int8 on the headline matrix, one GEMV per launch."""
+    K, N, S = 6912, 2560, 4096
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    rng = np.random.default_rng(0)
+    for M in (1, 4):
+        xs = ((0, "i8", sp.make_x_i8(1, M, K)), (1, "f16", rng.standard_normal((M, K)).astype(np.float16)),
+              (2, "f32", rng.standard_normal((M, K)).astype(np.float32)))
+        cb = sp.DeviceBuffer(4 * M * N)
+        for enc, split in (("delta", 32), ("u16", 32)):
+            w = sp.Weights.upload_delta(pos, neg, K, split) if enc == "delta" else sp.Weights.upload_u16(pos, neg, K, split)
+            n = copies_for(w.nbytes)
+            cps = [w] + [w.clone() for _ in range(n - 1)]
+            for act, name, X in xs:
+                xb = sp.DeviceBuffer.from_numpy(X)
+                sp.measure_gemv(cps[:1], act, xb, M, cb, 200, 0, st)
+                warm = min(sp.measure_gemv(cps[:1], act, xb, M, cb, 2000, 0, st) for _ in range(3))
+                sp.measure_gemv(cps, act, xb, M, cb, 2 * n, 0, st)
+                cold = min(sp.measure_gemv(cps, act, xb, M, cb, 2000, 0, st) for _ in range(3))
+                xb.free()
+                print("headline M=%d %s/%d %-3s activations: warm %6.2f us  cold %6.2f us" % (M, enc, split, name, warm, cold), flush=True)
+                rows.append({"shape": "headline", "M": M, "enc": "%s/%d" % (enc, split), "act": name,
+                             "warm_us": round(warm, 3), "cold_us": round(cold, 3)})
+            for c in cps:
+                c.free()
+        cb.free()
+
+
 def main(argv):
     which = argv[1] if len(argv) > 1 else "layer"
     info = sp.device_init(0)
@@ -188,6 +217,8 @@ def main(argv):
     elif which == "density":
         for S in (256, 512, 1024, 2048, 4096):
             run_shape("S=%d" % S, 6912, 2560, S, (1,), (32,), st, rows)
+    elif which == "float":
+        float_rows(st, rows)
     elif which == "q8":
         q8_rows(st, rows)
     elif which == "large":
@@ -195,7 +226,7 @@ def main(argv):
     elif which == "headline":
         run_shape("headline", 6912, 2560, 4096, (1, 4), (16, 32, 64), st, rows)
     else:
-        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged|density|q8")
+        sys.exit("usage: python -m sptmm_amd.sweep layer|large|headline|fused|ragged|density|float|q8")
     assert all(r.get("ok", True) for r in rows), "encodings disagree"
     print(json.dumps({"device": info["arch"], "rows": rows}))
 
