@@ -1,0 +1,72 @@
+"""Seeded random shapes through every list encoding, against the oracle's dense int8 product.
+
+Covers what the fixed-shape tests leave open: per-task counts that straddle the straight-line /
+ring kernel choice, tails of every length, empty tasks, every split, M around the 1/4/8 tile sizes.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import oracle
+import sptmm_amd as sp
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def device():
+    return sp.device_init(0)
+
+
+def cases(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        K = 16 * int(rng.integers(1, 400))
+        N = 16 * int(rng.integers(1, 24))
+        dens = float(rng.choice([0.0, 0.02, 0.1, 0.3, 0.6, 0.9, 1.0]))
+        bal = float(rng.uniform(0.2, 0.8))
+        M = int(rng.integers(1, 10))
+        out.append((K, N, dens * bal, dens * (1 - bal), M, int(rng.integers(0, 2**31))))
+    return out
+
+
+@pytest.mark.parametrize("kind,splits", [(sp.KIND_U16, (8, 16, 32, 64, 128, 256)), (sp.KIND_DELTA, (8, 16, 32, 64))])
+def test_ragged_random_shapes(kind, splits):
+    for i, (K, N, pp, pn, M, seed) in enumerate(cases(20240 + kind, 40)):
+        W = sp.generate_ternary_iid(K, N, seed, pp, pn)
+        X = oracle.make_x_i8(seed ^ 0x55, M, K)
+        want = oracle.dense_i8(X, W)
+        split = splits[i % len(splits)]
+        print("random ragged", kind, "K", K, "N", N, "p", round(pp, 3), round(pn, 3), "M", M, "split", split, flush=True)
+        sys.stdout.flush()
+        w = sp.Weights.upload_dense(W, kind, split)
+        got = w.matmul(X)
+        w.free()
+        assert (got == want).all(), (K, N, pp, pn, M, split)
+
+
+def test_balanced_random_shapes():
+    rng = np.random.default_rng(7)
+    for i in range(40):
+        split = int(rng.choice([8, 16, 32, 64, 128, 256]))
+        n_lane = int(rng.integers(1, 40))
+        half = split * n_lane
+        K = 16 * ((2 * half) // 16 + int(rng.integers(1, 60)))
+        if K >= 65536:
+            continue
+        N = 16 * int(rng.integers(1, 16))
+        M = int(rng.integers(1, 10))
+        _, pos, neg = sp.generate_ternary(K, N, 2 * half)
+        X = oracle.make_x_i8(i + 1, M, K)
+        want = oracle.sptmm_i8(X, pos, neg)
+        print("random balanced K", K, "N", N, "S", 2 * half, "split", split, "n_lane", n_lane, "M", M, flush=True)
+        sys.stdout.flush()
+        w = sp.Weights.upload_u16(pos, neg, K, split)
+        assert (w.matmul(X) == want).all(), ("u16", K, N, half, split, M)
+        w.free()
+        if split <= 64:
+            w = sp.Weights.upload_delta(pos, neg, K, split)
+            assert (w.matmul(X) == want).all(), ("delta", K, N, half, split, M, w.info["delta_bits"])
+            w.free()
