@@ -153,8 +153,14 @@ def main():
         buf = sp.DeviceBuffer(nb)
         buf.fill(1)
         best = min(sp.read_kernel(buf, nb, st, 20, wgs) for wgs in (256, 512, 4096) for _ in range(2))
-        buf.free()
         ceiling = {"bytes": nb, "us": round(best, 2), "gbps": round(nb / best / 1e3, 1)}
+        # and launched the way one GEMV per launch is: one stream's worth of bytes per launch, rotating over
+        # BATCH regions (HBM-cold) or staying on one (cache-warm) -- the floor under `single_launch`
+        one = nbytes // 16 * 16
+        cold1 = min(sp.read_kernel(buf, one, st, 2048, wgs, BATCH, one) for wgs in (256, 512, 1024))
+        warm1 = min(sp.read_kernel(buf, one, st, 2048, wgs) for wgs in (256, 512, 1024))
+        buf.free()
+        ceiling["per_launch_read"] = {"bytes": one, "cold_us": round(cold1, 3), "warm_us": round(warm1, 3)}
 
     others = {}
     if "others" in legs:

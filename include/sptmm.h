@@ -227,13 +227,16 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
  * evicts cached weight streams between cold-read timings and calibrates the
  * traffic counters. */
 int sptmm_copy_kernel(void *dst_dev, const void *src_dev, size_t bytes, void *stream);
-/* Streams `bytes` of a device buffer through the GEMV kernels' own load
+/* Streams `bytes` of device memory through the GEMV kernels' own load
  * instruction and throws the data away (sink_dev: 4 bytes of device memory):
  * `launches` timed launches after one untimed, mean microseconds per launch.
- * The read bandwidth this reaches is the practical ceiling below the 8 TB/s
- * datasheet figure.  workgroups <= 0 picks 4 per compute unit. */
-int sptmm_read_kernel(const void *src_dev, size_t bytes, void *sink_dev, int workgroups, int launches, void *stream,
-                      double *us_per_launch);
+ * Launch i reads the region at src_dev + (i % regions) * stride_bytes, so that
+ * enough regions defeat the last-level cache.  What this reaches is the
+ * practical ceiling below the 8 TB/s datasheet figure -- for one large read,
+ * and for one launch per GEMV-sized read.  workgroups <= 0 picks 4 per compute
+ * unit. */
+int sptmm_read_kernel(const void *src_dev, size_t bytes, size_t stride_bytes, int regions, void *sink_dev, int workgroups,
+                      int launches, void *stream, double *us_per_launch);
 
 #ifdef __cplusplus
 }

@@ -93,7 +93,8 @@ def lib() -> C.CDLL:
         L.sptmm_measure_gemv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                          C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         L.sptmm_copy_kernel.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
-        L.sptmm_read_kernel.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
+        L.sptmm_read_kernel.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                                        C.POINTER(C.c_double)]
         L.sptmm_make_x_i8.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p]
         L.sptmm_generate_ternary_iid.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_double, C.c_double, C.c_void_p]
         for n in ("sptmm_stream_create", "sptmm_event_create"):
@@ -352,12 +353,13 @@ def device_sync():
     _ck(lib().sptmm_device_sync())
 
 
-def read_kernel(src: DeviceBuffer, nbytes: int, stream: Stream, launches: int = 20, workgroups: int = 0) -> float:
-    """Mean microseconds per launch of a pure streaming read of `nbytes` of `src`."""
+def read_kernel(src: DeviceBuffer, nbytes: int, stream: Stream, launches: int = 20, workgroups: int = 0,
+                regions: int = 1, stride: int = 0) -> float:
+    """Mean microseconds per launch of a pure streaming read of `nbytes`; launch i reads region i % regions of `src`."""
     sink = DeviceBuffer(16)
     us = C.c_double()
     try:
-        _ck(lib().sptmm_read_kernel(src.ptr, nbytes, sink.ptr, workgroups, launches, stream.handle, C.byref(us)))
+        _ck(lib().sptmm_read_kernel(src.ptr, nbytes, stride, regions, sink.ptr, workgroups, launches, stream.handle, C.byref(us)))
     finally:
         sink.free()
     return us.value

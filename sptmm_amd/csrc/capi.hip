@@ -592,17 +592,20 @@ done:
     return rc;
 }
 
-int sptmm_read_kernel(const void *src, size_t bytes, void *sink, int workgroups, int launches, void *stream, double *us_per_launch)
+int sptmm_read_kernel(const void *src, size_t bytes, size_t stride_bytes, int regions, void *sink, int workgroups, int launches,
+                      void *stream, double *us_per_launch)
 {
-    if (!src || !sink || launches < 1 || !us_per_launch) return fail(SPTMM_ERR_INVALID, "bad argument");
+    if (!src || !sink || launches < 1 || regions < 1 || !us_per_launch) return fail(SPTMM_ERR_INVALID, "bad argument");
+    if (stride_bytes % 16) return fail(SPTMM_ERR_INVALID, "region stride must be a multiple of 16 bytes");
     if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_read_kernel needs a stream made by sptmm_stream_create");
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0, e1;
     HIP_TRY(hipEventCreate(&e0));
     HIP_TRY(hipEventCreate(&e1));
-    int rc = launch_read(src, bytes, sink, workgroups, stream);  // untimed first launch
+    auto region = [&](int i) { return (const uint8_t *)src + (size_t)(i % regions) * stride_bytes; };
+    int rc = launch_read(region(0), bytes, sink, workgroups, stream);  // untimed first launch
     hipError_t e = hipEventRecord(e0, st);
-    for (int i = 0; i < launches && rc == SPTMM_OK; ++i) rc = launch_read(src, bytes, sink, workgroups, stream);
+    for (int i = 0; i < launches && rc == SPTMM_OK; ++i) rc = launch_read(region(i + 1), bytes, sink, workgroups, stream);
     if (e == hipSuccess) e = hipEventRecord(e1, st);
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     float ms = 0.f;
