@@ -329,12 +329,8 @@ struct Round {
 typedef u32 v4u __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 stream_load(const uint4 *p)
 {
-#ifdef SPTMM_NO_NT
-    return *p;
-#else
     v4u t = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(p));
     return make_uint4(t.x, t.y, t.z, t.w);
-#endif
 }
 __device__ __forceinline__ Round load_round(const uint4 *wp, int r)
 {
@@ -422,10 +418,7 @@ struct ListsBody {
     static constexpr int SLOT = SLOT_OF;
     static constexpr int RING = 8;                    // rounds in flight on the generic path
     static constexpr int XMAX = VAR ? 2 : 0;          // ragged tasks on the straight-line path: full rounds beyond RF a task may have
-#ifndef SPTMM_EARLY
-#define SPTMM_EARLY 2
-#endif
-    static constexpr int EARLY = SPTMM_EARLY;         // rounds requested before the activation tile is complete
+    static constexpr int EARLY = 2;                   // rounds requested before the activation tile is complete
 
     static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, Sums<Act, MT> &acc)
     {
