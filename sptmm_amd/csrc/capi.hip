@@ -137,113 +137,125 @@ extern "C" {
 
 int sptmm_device_init(int device, sptmm_devinfo *out)
 {
-    int count = 0;
-    hipError_t e = hipGetDeviceCount(&count);
-    if (e != hipSuccess || count == 0) return fail(SPTMM_ERR_HIP, "no HIP device available (%s)", hipGetErrorString(e));
-    if (device < 0 || device >= count) return fail(SPTMM_ERR_INVALID, "device %d out of range (have %d)", device, count);
-    HIP_TRY(hipSetDevice(device));
-    if (out) {
-        hipDeviceProp_t pr;
-        HIP_TRY(hipGetDeviceProperties(&pr, device));
-        memset(out, 0, sizeof *out);
-        strncpy(out->name, pr.name, sizeof out->name - 1);
-        strncpy(out->arch, pr.gcnArchName, sizeof out->arch - 1);
-        out->compute_units = pr.multiProcessorCount;
-        out->wave_size = pr.warpSize;
-        out->lds_bytes_per_workgroup = (int)pr.sharedMemPerBlock;
-        out->l2_bytes = pr.l2CacheSize;
-        out->hbm_bytes = pr.totalGlobalMem;
-        out->peak_hbm_gbps = 8000.0;  // MI355X HBM3E, published
-    }
-    return SPTMM_OK;
+    return guarded([&]() -> int {
+        int count = 0;
+        hipError_t e = hipGetDeviceCount(&count);
+        if (e != hipSuccess || count == 0) return fail(SPTMM_ERR_HIP, "no HIP device available (%s)", hipGetErrorString(e));
+        if (device < 0 || device >= count) return fail(SPTMM_ERR_INVALID, "device %d out of range (have %d)", device, count);
+        HIP_TRY(hipSetDevice(device));
+        if (out) {
+            hipDeviceProp_t pr;
+            HIP_TRY(hipGetDeviceProperties(&pr, device));
+            memset(out, 0, sizeof *out);
+            strncpy(out->name, pr.name, sizeof out->name - 1);
+            strncpy(out->arch, pr.gcnArchName, sizeof out->arch - 1);
+            out->compute_units = pr.multiProcessorCount;
+            out->wave_size = pr.warpSize;
+            out->lds_bytes_per_workgroup = (int)pr.sharedMemPerBlock;
+            out->l2_bytes = pr.l2CacheSize;
+            out->hbm_bytes = pr.totalGlobalMem;
+            out->peak_hbm_gbps = 8000.0;  // MI355X HBM3E, published
+        }
+        return SPTMM_OK;
+    });
 }
 
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out)
 {
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (int rc = check_shape(K, N, S)) return rc;
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
-    std::vector<uint8_t> host(sptmm_pack_u16_bytes(N, S, split_k));
-    if (int rc = sptmm_pack_u16(pos, neg, K, N, S, split_k, host.data())) return rc;
-    sptmm_weights *w = new (std::nothrow) sptmm_weights();
-    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{SPTMM_KIND_U16, K, N, S, split_k, 0, 0, 0, (uint64_t)S * N};
-    w->index_shift = u16_index_shift(K);
-    w->geo = g;
-    return finish_upload(w, host, out);
+    return guarded([&]() -> int {
+        if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (int rc = check_shape(K, N, S)) return rc;
+        Geometry g;
+        if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
+        std::vector<uint8_t> host(sptmm_pack_u16_bytes(N, S, split_k));
+        if (int rc = sptmm_pack_u16(pos, neg, K, N, S, split_k, host.data())) return rc;
+        sptmm_weights *w = new (std::nothrow) sptmm_weights();
+        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        w->info = sptmm_winfo{SPTMM_KIND_U16, K, N, S, split_k, 0, 0, 0, (uint64_t)S * N};
+        w->index_shift = u16_index_shift(K);
+        w->geo = g;
+        return finish_upload(w, host, out);
+    });
 }
 
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out)
 {
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (int rc = check_shape(K, N, S)) return rc;
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
-    int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
-    if (bits < 0) return bits;
-    std::vector<uint8_t> host(sptmm_pack_delta_bytes(N, S, split_k, bits));
-    if (int rc = sptmm_pack_delta(pos, neg, K, N, S, split_k, bits, host.data())) return rc;
-    sptmm_weights *w = new (std::nothrow) sptmm_weights();
-    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{SPTMM_KIND_DELTA, K, N, S, split_k, bits, 0, 0, (uint64_t)S * N};
-    w->geo = g;
-    return finish_upload(w, host, out);
+    return guarded([&]() -> int {
+        if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (int rc = check_shape(K, N, S)) return rc;
+        Geometry g;
+        if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
+        int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
+        if (bits < 0) return bits;
+        std::vector<uint8_t> host(sptmm_pack_delta_bytes(N, S, split_k, bits));
+        if (int rc = sptmm_pack_delta(pos, neg, K, N, S, split_k, bits, host.data())) return rc;
+        sptmm_weights *w = new (std::nothrow) sptmm_weights();
+        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        w->info = sptmm_winfo{SPTMM_KIND_DELTA, K, N, S, split_k, bits, 0, 0, (uint64_t)S * N};
+        w->geo = g;
+        return finish_upload(w, host, out);
+    });
 }
 
 int sptmm_weights_upload_i2s(const int8_t *W, int K, int N, sptmm_weights **out)
 {
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    size_t bytes = sptmm_pack_i2s_bytes(K, N);
-    if (!bytes) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
-    std::vector<uint8_t> host(bytes);
-    if (int rc = sptmm_pack_i2s(W, K, N, host.data())) return rc;
-    sptmm_weights *w = new (std::nothrow) sptmm_weights();
-    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{SPTMM_KIND_I2S, K, N, 0, 0, 0, 0, 0, 0};
-    w->geo = Geometry{};
-    return finish_upload(w, host, out);
+    return guarded([&]() -> int {
+        if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        size_t bytes = sptmm_pack_i2s_bytes(K, N);
+        if (!bytes) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
+        std::vector<uint8_t> host(bytes);
+        if (int rc = sptmm_pack_i2s(W, K, N, host.data())) return rc;
+        sptmm_weights *w = new (std::nothrow) sptmm_weights();
+        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        w->info = sptmm_winfo{SPTMM_KIND_I2S, K, N, 0, 0, 0, 0, 0, 0};
+        w->geo = Geometry{};
+        return finish_upload(w, host, out);
+    });
 }
 
 int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int split_k, sptmm_weights **out)
 {
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (kind == SPTMM_KIND_I2S) return sptmm_weights_upload_i2s(W, K, N, out);
-    int bits = 0, n_min = 0, n_max = 0;
-    size_t read_bytes = 0;
-    uint64_t nnz = 0;
-    const size_t bytes = sptmm_pack_ragged_bytes(W, K, N, kind, split_k, &bits, &read_bytes, &n_min, &n_max, &nnz);
-    if (!bytes) return SPTMM_ERR_INVALID;  // message set by the planner
-    std::vector<uint8_t> host(bytes);
-    if (int rc = sptmm_pack_ragged(W, K, N, kind, split_k, bits, host.data())) return rc;
-    sptmm_weights *w = new (std::nothrow) sptmm_weights();
-    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{kind, K, N, 0, split_k, bits, read_bytes, 1, nnz};
-    if (int rc = make_ragged_geometry(N, split_k, 256, &w->geo)) {
-        delete w;
-        return rc;
-    }
-    w->counts_bytes = (int)ragged_counts_bytes(w->geo.tasks);
-    w->task_stride = (int)((bytes - w->counts_bytes) / w->geo.tasks);
-    w->n_min = n_min;
-    w->n_max = n_max;
-    w->index_shift = kind == SPTMM_KIND_U16 ? ragged_index_shift(K) : 0;
-    return finish_upload(w, host, out);
+    return guarded([&]() -> int {
+        if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (kind == SPTMM_KIND_I2S) return sptmm_weights_upload_i2s(W, K, N, out);
+        int bits = 0, n_min = 0, n_max = 0;
+        size_t read_bytes = 0;
+        uint64_t nnz = 0;
+        const size_t bytes = sptmm_pack_ragged_bytes(W, K, N, kind, split_k, &bits, &read_bytes, &n_min, &n_max, &nnz);
+        if (!bytes) return SPTMM_ERR_INVALID;  // message set by the planner
+        std::vector<uint8_t> host(bytes);
+        if (int rc = sptmm_pack_ragged(W, K, N, kind, split_k, bits, host.data())) return rc;
+        sptmm_weights *w = new (std::nothrow) sptmm_weights();
+        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        w->info = sptmm_winfo{kind, K, N, 0, split_k, bits, read_bytes, 1, nnz};
+        if (int rc = make_ragged_geometry(N, split_k, 256, &w->geo)) {
+            delete w;
+            return rc;
+        }
+        w->counts_bytes = (int)ragged_counts_bytes(w->geo.tasks);
+        w->task_stride = (int)((bytes - w->counts_bytes) / w->geo.tasks);
+        w->n_min = n_min;
+        w->n_max = n_max;
+        w->index_shift = kind == SPTMM_KIND_U16 ? ragged_index_shift(K) : 0;
+        return finish_upload(w, host, out);
+    });
 }
 
 int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out)
 {
-    if (!w || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    sptmm_weights *c = new (std::nothrow) sptmm_weights(*w);
-    if (!c) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    hipError_t e = hipMalloc(&c->dev, w->bytes);
-    if (e == hipSuccess) e = hipMemcpy(c->dev, w->dev, w->bytes, hipMemcpyDeviceToDevice);
-    if (e != hipSuccess) {
-        delete c;
-        return hip_fail(e, "clone weight stream");
-    }
-    *out = c;
-    return SPTMM_OK;
+    return guarded([&]() -> int {
+        if (!w || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        sptmm_weights *c = new (std::nothrow) sptmm_weights(*w);
+        if (!c) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        hipError_t e = hipMalloc(&c->dev, w->bytes);
+        if (e == hipSuccess) e = hipMemcpy(c->dev, w->dev, w->bytes, hipMemcpyDeviceToDevice);
+        if (e != hipSuccess) {
+            delete c;
+            return hip_fail(e, "clone weight stream");
+        }
+        *out = c;
+        return SPTMM_OK;
+    });
 }
 
 void sptmm_weights_free(sptmm_weights *w)
@@ -292,98 +304,102 @@ uint64_t file_checksum(FileHeader h, const std::vector<uint8_t> &stream)
 
 int sptmm_weights_save(const sptmm_weights *w, const char *path)
 {
-    if (!w || !path) return fail(SPTMM_ERR_INVALID, "null pointer");
-    std::vector<uint8_t> host(w->bytes);
-    HIP_TRY(hipMemcpy(host.data(), w->dev, w->bytes, hipMemcpyDeviceToHost));
-    FileHeader h{};
-    memcpy(h.magic, FILE_MAGIC, 8);
-    h.header_bytes = (uint32_t)sizeof h;
-    h.version = 1;
-    const sptmm_winfo &i = w->info;
-    const Geometry &g = w->geo;
-    h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = i.ragged;
-    h.half = g.half, h.L = g.L, h.G = g.G, h.W = g.W, h.n_lane = g.n_lane, h.tasks = g.tasks;
-    h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max, h.index_shift = w->index_shift;
-    h.nnz = i.nnz, h.read_bytes = i.stream_bytes, h.stream_bytes = w->bytes;
-    h.fnv1a = file_checksum(h, host);
-    FILE *f = fopen(path, "wb");
-    if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s for writing", path);
-    const bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(host.data(), 1, host.size(), f) == host.size();
-    if (fclose(f) != 0 || !ok) return fail(SPTMM_ERR_INVALID, "short write to %s", path);
-    return SPTMM_OK;
+    return guarded([&]() -> int {
+        if (!w || !path) return fail(SPTMM_ERR_INVALID, "null pointer");
+        std::vector<uint8_t> host(w->bytes);
+        HIP_TRY(hipMemcpy(host.data(), w->dev, w->bytes, hipMemcpyDeviceToHost));
+        FileHeader h{};
+        memcpy(h.magic, FILE_MAGIC, 8);
+        h.header_bytes = (uint32_t)sizeof h;
+        h.version = 1;
+        const sptmm_winfo &i = w->info;
+        const Geometry &g = w->geo;
+        h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = i.ragged;
+        h.half = g.half, h.L = g.L, h.G = g.G, h.W = g.W, h.n_lane = g.n_lane, h.tasks = g.tasks;
+        h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max, h.index_shift = w->index_shift;
+        h.nnz = i.nnz, h.read_bytes = i.stream_bytes, h.stream_bytes = w->bytes;
+        h.fnv1a = file_checksum(h, host);
+        FILE *f = fopen(path, "wb");
+        if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s for writing", path);
+        const bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(host.data(), 1, host.size(), f) == host.size();
+        if (fclose(f) != 0 || !ok) return fail(SPTMM_ERR_INVALID, "short write to %s", path);
+        return SPTMM_OK;
+    });
 }
 
 int sptmm_weights_load(const char *path, sptmm_weights **out)
 {
-    if (!path || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    FILE *f = fopen(path, "rb");
-    if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s", path);
-    FileHeader h{};
-    std::vector<uint8_t> host;
-    int rc = SPTMM_OK;
-    if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || h.version != 1)
-        rc = fail(SPTMM_ERR_INVALID, "%s is not a weight file of this library", path);
-    // every field the kernels index with is checked against the stream size before anything is uploaded
-    if (!rc) {
-        Geometry g{};
-        size_t want = 0;
-        if (h.kind == SPTMM_KIND_I2S) {
-            want = sptmm_pack_i2s_bytes(h.K, h.N);
-        } else if (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA) {
-            const int max_split = h.kind == SPTMM_KIND_U16 ? 256 : 64;
-            const bool gaps = h.kind == SPTMM_KIND_DELTA;
-            if (gaps ? (h.delta_bits != 8 && h.delta_bits != 16) : h.delta_bits != 0) {
-                rc = fail(SPTMM_ERR_INVALID, "%s: bad gap width", path);
-            } else if (h.ragged) {
-                const int esz = gaps ? h.delta_bits / 8 : 2;
-                if (h.K <= 0 || h.N <= 0 || h.K % 16 || h.N % 16 || h.K + 64 > 65535 || make_ragged_geometry(h.N, h.split_k, max_split, &g) ||
-                    h.n_min < 1 || h.n_max < h.n_min || h.n_max > 65535 || h.counts_bytes != (int)ragged_counts_bytes(g.tasks) ||
-                    h.task_stride != (gaps ? 256 : 0) + 128 * esz * h.n_max ||
-                    h.index_shift != (gaps ? 0 : ragged_index_shift(h.K)))
-                    rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent ragged stream header", path);
-                else
-                    want = (size_t)h.counts_bytes + (size_t)h.task_stride * g.tasks;
+    return guarded([&]() -> int {
+        if (!path || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        FILE *f = fopen(path, "rb");
+        if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s", path);
+        FileHeader h{};
+        std::vector<uint8_t> host;
+        int rc = SPTMM_OK;
+        if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || h.version != 1)
+            rc = fail(SPTMM_ERR_INVALID, "%s is not a weight file of this library", path);
+        // every field the kernels index with is checked against the stream size before anything is uploaded
+        if (!rc) {
+            Geometry g{};
+            size_t want = 0;
+            if (h.kind == SPTMM_KIND_I2S) {
+                want = sptmm_pack_i2s_bytes(h.K, h.N);
+            } else if (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA) {
+                const int max_split = h.kind == SPTMM_KIND_U16 ? 256 : 64;
+                const bool gaps = h.kind == SPTMM_KIND_DELTA;
+                if (gaps ? (h.delta_bits != 8 && h.delta_bits != 16) : h.delta_bits != 0) {
+                    rc = fail(SPTMM_ERR_INVALID, "%s: bad gap width", path);
+                } else if (h.ragged) {
+                    const int esz = gaps ? h.delta_bits / 8 : 2;
+                    if (h.K <= 0 || h.N <= 0 || h.K % 16 || h.N % 16 || h.K + 64 > 65535 || make_ragged_geometry(h.N, h.split_k, max_split, &g) ||
+                        h.n_min < 1 || h.n_max < h.n_min || h.n_max > 65535 || h.counts_bytes != (int)ragged_counts_bytes(g.tasks) ||
+                        h.task_stride != (gaps ? 256 : 0) + 128 * esz * h.n_max ||
+                        h.index_shift != (gaps ? 0 : ragged_index_shift(h.K)))
+                        rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent ragged stream header", path);
+                    else
+                        want = (size_t)h.counts_bytes + (size_t)h.task_stride * g.tasks;
+                } else {
+                    if (check_shape(h.K, h.N, h.S) || make_geometry(h.N, h.S, h.split_k, max_split, &g) ||
+                        h.index_shift != (gaps ? 0 : u16_index_shift(h.K)))
+                        rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent stream header", path);
+                    else
+                        want = gaps ? sptmm_pack_delta_bytes(h.N, h.S, h.split_k, h.delta_bits) : sptmm_pack_u16_bytes(h.N, h.S, h.split_k);
+                }
+                if (!rc && (g.half != h.half || g.L != h.L || g.G != h.G || g.W != h.W || g.n_lane != h.n_lane || g.tasks != h.tasks))
+                    rc = fail(SPTMM_ERR_INVALID, "%s: geometry does not match the shape", path);
             } else {
-                if (check_shape(h.K, h.N, h.S) || make_geometry(h.N, h.S, h.split_k, max_split, &g) ||
-                    h.index_shift != (gaps ? 0 : u16_index_shift(h.K)))
-                    rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent stream header", path);
-                else
-                    want = gaps ? sptmm_pack_delta_bytes(h.N, h.S, h.split_k, h.delta_bits) : sptmm_pack_u16_bytes(h.N, h.S, h.split_k);
+                rc = fail(SPTMM_ERR_INVALID, "%s: unknown stream kind %d", path, h.kind);
             }
-            if (!rc && (g.half != h.half || g.L != h.L || g.G != h.G || g.W != h.W || g.n_lane != h.n_lane || g.tasks != h.tasks))
-                rc = fail(SPTMM_ERR_INVALID, "%s: geometry does not match the shape", path);
-        } else {
-            rc = fail(SPTMM_ERR_INVALID, "%s: unknown stream kind %d", path, h.kind);
+            if (!rc && (want == 0 || want != h.stream_bytes)) rc = fail(SPTMM_ERR_INVALID, "%s: stream size does not match the shape", path);
         }
-        if (!rc && (want == 0 || want != h.stream_bytes)) rc = fail(SPTMM_ERR_INVALID, "%s: stream size does not match the shape", path);
-    }
-    if (!rc) {
-        host.resize(h.stream_bytes);
-        if (fread(host.data(), 1, host.size(), f) != host.size() || fgetc(f) != EOF)
-            rc = fail(SPTMM_ERR_INVALID, "%s: truncated or oversized file", path);
-        else if (file_checksum(h, host) != h.fnv1a)
-            rc = fail(SPTMM_ERR_INVALID, "%s: checksum mismatch", path);
-    }
-    fclose(f);
-    if (rc) return rc;
-    if (h.ragged && (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA)) {
-        // the per-task counts are what the kernel trusts most: keep them inside [n_min, n_max]
-        const uint32_t *pre = (const uint32_t *)host.data();
-        const uint16_t *counts = (const uint16_t *)(host.data() + 16);
-        bool ok = pre[0] == RAGGED_MAGIC && pre[1] == (uint32_t)h.tasks && pre[2] == (uint32_t)h.n_max && pre[3] == (uint32_t)h.n_min;
-        for (int t = 0; ok && t < h.tasks; ++t) ok = counts[t] >= h.n_min && counts[t] <= h.n_max;
-        if (!ok) return fail(SPTMM_ERR_INVALID, "%s: corrupt count table", path);
-    }
-    sptmm_weights *w = new (std::nothrow) sptmm_weights();
-    if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-    w->info = sptmm_winfo{h.kind, h.K, h.N, h.S, h.split_k, h.delta_bits, h.read_bytes, h.ragged, h.nnz};
-    w->geo = Geometry{h.N, h.half, h.split_k, h.L, h.G, h.W, h.n_lane, h.tasks};
-    w->task_stride = h.task_stride;
-    w->counts_bytes = h.counts_bytes;
-    w->n_min = h.n_min;
-    w->n_max = h.n_max;
-    w->index_shift = h.index_shift;
-    return finish_upload(w, host, out);
+        if (!rc) {
+            host.resize(h.stream_bytes);
+            if (fread(host.data(), 1, host.size(), f) != host.size() || fgetc(f) != EOF)
+                rc = fail(SPTMM_ERR_INVALID, "%s: truncated or oversized file", path);
+            else if (file_checksum(h, host) != h.fnv1a)
+                rc = fail(SPTMM_ERR_INVALID, "%s: checksum mismatch", path);
+        }
+        fclose(f);
+        if (rc) return rc;
+        if (h.ragged && (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA)) {
+            // the per-task counts are what the kernel trusts most: keep them inside [n_min, n_max]
+            const uint32_t *pre = (const uint32_t *)host.data();
+            const uint16_t *counts = (const uint16_t *)(host.data() + 16);
+            bool ok = pre[0] == RAGGED_MAGIC && pre[1] == (uint32_t)h.tasks && pre[2] == (uint32_t)h.n_max && pre[3] == (uint32_t)h.n_min;
+            for (int t = 0; ok && t < h.tasks; ++t) ok = counts[t] >= h.n_min && counts[t] <= h.n_max;
+            if (!ok) return fail(SPTMM_ERR_INVALID, "%s: corrupt count table", path);
+        }
+        sptmm_weights *w = new (std::nothrow) sptmm_weights();
+        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        w->info = sptmm_winfo{h.kind, h.K, h.N, h.S, h.split_k, h.delta_bits, h.read_bytes, h.ragged, h.nnz};
+        w->geo = Geometry{h.N, h.half, h.split_k, h.L, h.G, h.W, h.n_lane, h.tasks};
+        w->task_stride = h.task_stride;
+        w->counts_bytes = h.counts_bytes;
+        w->n_min = h.n_min;
+        w->n_max = h.n_max;
+        w->index_shift = h.index_shift;
+        return finish_upload(w, host, out);
+    });
 }
 
 int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X, int M, int32_t *C, void *stream)
@@ -394,22 +410,24 @@ int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X, int M, int32_t *C, vo
 int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X, int32_t *const *C, int count, int M,
                           void *stream)
 {
-    if (!ws || !X || !C || count < 1) return fail(SPTMM_ERR_INVALID, "bad argument");
-    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
-    std::vector<const void *> wp(count), xp(count);
-    std::vector<void *> cp(count);
-    for (int i = 0; i < count; ++i) {
-        if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
-        const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
-        if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
-            a.ragged != b.ragged || ws[0]->task_stride != ws[i]->task_stride ||
-            ws[0]->n_min != ws[i]->n_min)
-            return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);
-        wp[i] = ws[i]->dev;
-        xp[i] = X[i];
-        cp[i] = C[i];
-    }
-    return gemv_common(ws[0], X[0], M, C[0], stream, ACT_I8, count, wp.data(), xp.data(), cp.data());
+    return guarded([&]() -> int {
+        if (!ws || !X || !C || count < 1) return fail(SPTMM_ERR_INVALID, "bad argument");
+        if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+        std::vector<const void *> wp(count), xp(count);
+        std::vector<void *> cp(count);
+        for (int i = 0; i < count; ++i) {
+            if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
+            const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
+            if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
+                a.ragged != b.ragged || ws[0]->task_stride != ws[i]->task_stride ||
+                ws[0]->n_min != ws[i]->n_min)
+                return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);
+            wp[i] = ws[i]->dev;
+            xp[i] = X[i];
+            cp[i] = C[i];
+        }
+        return gemv_common(ws[0], X[0], M, C[0], stream, ACT_I8, count, wp.data(), xp.data(), cp.data());
+    });
 }
 
 int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X, int x_type, int M, float w_scale, float *Y, void *stream)

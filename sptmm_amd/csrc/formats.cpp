@@ -6,6 +6,7 @@
 #include <array>
 #include <cstdio>
 #include <cstring>
+#include <exception>
 #include <thread>
 #include <vector>
 
@@ -113,18 +114,26 @@ static inline Place place(const Geometry &g, int c, int i, bool contiguous)
 }
 
 template <class F>
-static void parallel_columns(int N, F f)
+static void parallel_columns(int n, F f)
 {
+    // worker threads; the first exception any of them meets is rethrown on the calling thread
     unsigned hw = std::thread::hardware_concurrency();
     int nt = (int)std::min<unsigned>(hw ? hw : 1, 16);
-    if (N < 64) nt = 1;
+    if (n < 64) nt = 1;
     std::vector<std::thread> th;
+    std::vector<std::exception_ptr> err(nt);
     for (int t = 0; t < nt; ++t)
-        th.emplace_back([=] {
-            int c0 = (int)((long)N * t / nt), c1 = (int)((long)N * (t + 1) / nt);
-            for (int c = c0; c < c1; ++c) f(c);
+        th.emplace_back([=, &err] {
+            try {
+                int i0 = (int)((long)n * t / nt), i1 = (int)((long)n * (t + 1) / nt);
+                for (int i = i0; i < i1; ++i) f(i);
+            } catch (...) {
+                err[t] = std::current_exception();
+            }
         });
     for (auto &t : th) t.join();
+    for (auto &e : err)
+        if (e) std::rethrow_exception(e);
 }
 
 static inline uint32_t xorshift32(uint32_t &s)
@@ -146,57 +155,61 @@ const char *sptmm_version(void) { return "sptmm-mi355x 0.1 (gfx950)"; }
 
 int sptmm_lists_from_dense(const int8_t *W, int K, int N, int S, uint16_t *pos, uint16_t *neg)
 {
-    if (int rc = check_shape(K, N, S)) return rc;
-    if (!W || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const int half = S / 2;
-    std::vector<int> bad(N, 0);
-    parallel_columns(N, [&](int c) {
-        const int8_t *w = W + (size_t)c * K;
-        int np = 0, nn = 0;
-        for (int r = 0; r < K; ++r) {
-            if (w[r] == 1) {
-                if (np < half) pos[(size_t)c * half + np] = (uint16_t)r;
-                ++np;
-            } else if (w[r] == -1) {
-                if (nn < half) neg[(size_t)c * half + nn] = (uint16_t)r;
-                ++nn;
-            } else if (w[r] != 0) {
-                bad[c] = 1;
+    return guarded([&]() -> int {
+        if (int rc = check_shape(K, N, S)) return rc;
+        if (!W || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+        const int half = S / 2;
+        std::vector<int> bad(N, 0);
+        parallel_columns(N, [&](int c) {
+            const int8_t *w = W + (size_t)c * K;
+            int np = 0, nn = 0;
+            for (int r = 0; r < K; ++r) {
+                if (w[r] == 1) {
+                    if (np < half) pos[(size_t)c * half + np] = (uint16_t)r;
+                    ++np;
+                } else if (w[r] == -1) {
+                    if (nn < half) neg[(size_t)c * half + nn] = (uint16_t)r;
+                    ++nn;
+                } else if (w[r] != 0) {
+                    bad[c] = 1;
+                }
             }
-        }
-        if (np != half || nn != half) bad[c] = 1;
+            if (np != half || nn != half) bad[c] = 1;
+        });
+        for (int c = 0; c < N; ++c)
+            if (bad[c]) return fail(SPTMM_ERR_INVALID, "W matrix corrupt: column %d is not ternary with S/2 entries per sign", c);
+        return SPTMM_OK;
     });
-    for (int c = 0; c < N; ++c)
-        if (bad[c]) return fail(SPTMM_ERR_INVALID, "W matrix corrupt: column %d is not ternary with S/2 entries per sign", c);
-    return SPTMM_OK;
 }
 
 int sptmm_generate_ternary(int K, int N, int S, int8_t *W, uint16_t *pos, uint16_t *neg)
 {
-    if (int rc = check_shape(K, N, S)) return rc;
-    if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const int half = S / 2;
-    parallel_columns(N, [&](int c) {
-        std::vector<int8_t> local;
-        int8_t *w;
-        if (W) {
-            w = W + (size_t)c * K;
-        } else {
-            local.resize(K);
-            w = local.data();
-        }
-        std::fill(w, w + half, (int8_t)-1);
-        std::fill(w + half, w + S, (int8_t)1);
-        std::fill(w + S, w + K, (int8_t)0);
-        uint32_t st = 0xCAFEBABEu ^ (uint32_t)c;
-        for (uint32_t i = (uint32_t)K - 1; i > 0; --i) std::swap(w[i], w[xorshift32(st) % (i + 1)]);
-        uint16_t *p = pos + (size_t)c * half, *q = neg + (size_t)c * half;
-        for (int r = 0; r < K; ++r) {
-            if (w[r] > 0) *p++ = (uint16_t)r;
-            if (w[r] < 0) *q++ = (uint16_t)r;
-        }
+    return guarded([&]() -> int {
+        if (int rc = check_shape(K, N, S)) return rc;
+        if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+        const int half = S / 2;
+        parallel_columns(N, [&](int c) {
+            std::vector<int8_t> local;
+            int8_t *w;
+            if (W) {
+                w = W + (size_t)c * K;
+            } else {
+                local.resize(K);
+                w = local.data();
+            }
+            std::fill(w, w + half, (int8_t)-1);
+            std::fill(w + half, w + S, (int8_t)1);
+            std::fill(w + S, w + K, (int8_t)0);
+            uint32_t st = 0xCAFEBABEu ^ (uint32_t)c;
+            for (uint32_t i = (uint32_t)K - 1; i > 0; --i) std::swap(w[i], w[xorshift32(st) % (i + 1)]);
+            uint16_t *p = pos + (size_t)c * half, *q = neg + (size_t)c * half;
+            for (int r = 0; r < K; ++r) {
+                if (w[r] > 0) *p++ = (uint16_t)r;
+                if (w[r] < 0) *q++ = (uint16_t)r;
+            }
+        });
+        return SPTMM_OK;
     });
-    return SPTMM_OK;
 }
 
 int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X)
@@ -418,83 +431,87 @@ extern "C" {
 
 int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out)
 {
-    if (int rc = check_shape(K, N, S)) return rc;
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
-    if (!out || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    for (size_t i = 0, n = (size_t)N * g.half; i < n; ++i)
-        if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
-    const int sh = u16_index_shift(K);
-    const size_t task_bytes = (size_t)256 * g.n_lane;
-    uint8_t *base = (uint8_t *)out;
-    auto put = [&](int task, int lane, int slot, int sign, uint16_t k) {
-        *(uint16_t *)(base + task * task_bytes + slot_offset(g.n_lane, 2, sign, lane, slot)) = (uint16_t)(k << sh);
-    };
-    // groups of columns that share half-wavefronts: one column when L >= 32, else 32/L columns
-    const int group = g.L >= 32 ? 1 : 32 / g.L;
-    parallel_columns(N / group, [&](int gi) {
-        for (int sign = 0; sign < 2; ++sign) {
-            const uint16_t *lists = sign ? neg : pos;
-            if (g.L == 64) {
-                // deal the column's entries, bank by bank, round-robin over its 2*W half-wavefronts
-                const int c = gi, nd = 2 * g.W;
-                std::vector<uint16_t> e(lists + (size_t)c * g.half, lists + (size_t)(c + 1) * g.half);
-                std::stable_sort(e.begin(), e.end(), [](uint16_t x, uint16_t y) { return (x & 31) < (y & 31); });
-                std::vector<Domain> dom(nd);
-                for (int d = 0; d < nd; ++d) {
-                    dom[d].owners = 1;
-                    dom[d].lanes = 32;
-                    dom[d].n = g.n_lane;
-                    dom[d].entries.resize(1);
-                }
-                for (int i = 0; i < g.half; ++i) dom[i % nd].entries[0].push_back(e[i]);
-                for (int d = 0; d < nd; ++d) {
-                    schedule(dom[d]);
-                    for (int slot = 0; slot < g.n_lane; ++slot)
-                        for (int l = 0; l < 32; ++l)
-                            put(c * g.W + d / 2, 32 * (d % 2) + l, slot, sign, dom[d].cell[0][(size_t)slot * 32 + l]);
-                }
-            } else {
-                Domain d;
-                d.owners = group;
-                d.lanes = g.L >= 32 ? 32 : g.L;
-                d.n = g.n_lane;
-                d.entries.resize(group);
-                for (int o = 0; o < group; ++o) {
-                    const int c = gi * group + o;
-                    d.entries[o].assign(lists + (size_t)c * g.half, lists + (size_t)(c + 1) * g.half);
-                }
-                schedule(d);
-                for (int o = 0; o < group; ++o) {
-                    const int c = gi * group + o, task = c / g.G, l0 = (c % g.G) * g.L;
-                    for (int slot = 0; slot < g.n_lane; ++slot)
-                        for (int l = 0; l < d.lanes; ++l) put(task, l0 + l, slot, sign, d.cell[o][(size_t)slot * d.lanes + l]);
+    return guarded([&]() -> int {
+        if (int rc = check_shape(K, N, S)) return rc;
+        Geometry g;
+        if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
+        if (!out || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+        for (size_t i = 0, n = (size_t)N * g.half; i < n; ++i)
+            if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
+        const int sh = u16_index_shift(K);
+        const size_t task_bytes = (size_t)256 * g.n_lane;
+        uint8_t *base = (uint8_t *)out;
+        auto put = [&](int task, int lane, int slot, int sign, uint16_t k) {
+            *(uint16_t *)(base + task * task_bytes + slot_offset(g.n_lane, 2, sign, lane, slot)) = (uint16_t)(k << sh);
+        };
+        // groups of columns that share half-wavefronts: one column when L >= 32, else 32/L columns
+        const int group = g.L >= 32 ? 1 : 32 / g.L;
+        parallel_columns(N / group, [&](int gi) {
+            for (int sign = 0; sign < 2; ++sign) {
+                const uint16_t *lists = sign ? neg : pos;
+                if (g.L == 64) {
+                    // deal the column's entries, bank by bank, round-robin over its 2*W half-wavefronts
+                    const int c = gi, nd = 2 * g.W;
+                    std::vector<uint16_t> e(lists + (size_t)c * g.half, lists + (size_t)(c + 1) * g.half);
+                    std::stable_sort(e.begin(), e.end(), [](uint16_t x, uint16_t y) { return (x & 31) < (y & 31); });
+                    std::vector<Domain> dom(nd);
+                    for (int d = 0; d < nd; ++d) {
+                        dom[d].owners = 1;
+                        dom[d].lanes = 32;
+                        dom[d].n = g.n_lane;
+                        dom[d].entries.resize(1);
+                    }
+                    for (int i = 0; i < g.half; ++i) dom[i % nd].entries[0].push_back(e[i]);
+                    for (int d = 0; d < nd; ++d) {
+                        schedule(dom[d]);
+                        for (int slot = 0; slot < g.n_lane; ++slot)
+                            for (int l = 0; l < 32; ++l)
+                                put(c * g.W + d / 2, 32 * (d % 2) + l, slot, sign, dom[d].cell[0][(size_t)slot * 32 + l]);
+                    }
+                } else {
+                    Domain d;
+                    d.owners = group;
+                    d.lanes = g.L >= 32 ? 32 : g.L;
+                    d.n = g.n_lane;
+                    d.entries.resize(group);
+                    for (int o = 0; o < group; ++o) {
+                        const int c = gi * group + o;
+                        d.entries[o].assign(lists + (size_t)c * g.half, lists + (size_t)(c + 1) * g.half);
+                    }
+                    schedule(d);
+                    for (int o = 0; o < group; ++o) {
+                        const int c = gi * group + o, task = c / g.G, l0 = (c % g.G) * g.L;
+                        for (int slot = 0; slot < g.n_lane; ++slot)
+                            for (int l = 0; l < d.lanes; ++l) put(task, l0 + l, slot, sign, d.cell[o][(size_t)slot * d.lanes + l]);
+                    }
                 }
             }
-        }
+        });
+        return SPTMM_OK;
     });
-    return SPTMM_OK;
 }
 
 int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint16_t *pos, uint16_t *neg)
 {
-    if (int rc = check_shape(K, N, S)) return rc;
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
-    if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const int sh = u16_index_shift(K);
-    const size_t task_bytes = (size_t)256 * g.n_lane;
-    const uint8_t *base = (const uint8_t *)packed;
-    parallel_columns(N, [&](int c) {
-        for (int sign = 0; sign < 2; ++sign) {
-            uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
-            for_cells(g, c, [&](int task, int lane, int slot, int i) {
-                lst[i] = (uint16_t)(*(const uint16_t *)(base + task * task_bytes + slot_offset(g.n_lane, 2, sign, lane, slot)) >> sh);
-            });
-            std::sort(lst, lst + g.half);
-        }
+    return guarded([&]() -> int {
+        if (int rc = check_shape(K, N, S)) return rc;
+        Geometry g;
+        if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
+        if (!packed || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+        const int sh = u16_index_shift(K);
+        const size_t task_bytes = (size_t)256 * g.n_lane;
+        const uint8_t *base = (const uint8_t *)packed;
+        parallel_columns(N, [&](int c) {
+            for (int sign = 0; sign < 2; ++sign) {
+                uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
+                for_cells(g, c, [&](int task, int lane, int slot, int i) {
+                    lst[i] = (uint16_t)(*(const uint16_t *)(base + task * task_bytes + slot_offset(g.n_lane, 2, sign, lane, slot)) >> sh);
+                });
+                std::sort(lst, lst + g.half);
+            }
+        });
+        return SPTMM_OK;
     });
-    return SPTMM_OK;
 }
 
 // ---------------------------------------------------------------- gap streams
@@ -506,20 +523,22 @@ int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint1
 // which keeps the lanes of a half-wavefront on different LDS banks.
 int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int split_k)
 {
-    Geometry g;
-    if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
-    if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
-    for (int sign = 0; sign < 2; ++sign) {
-        const uint16_t *l = sign ? neg : pos;
-        for (int c = 0; c < N; ++c)
-            for (int i = 1; i < g.half; ++i) {
-                if (i % g.n_lane == 0) continue;  // run start: absolute
-                size_t o = (size_t)c * g.half + i;
-                if (l[o] <= l[o - 1]) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending");
-                if (l[o] - l[o - 1] > 127) return 16;
-            }
-    }
-    return 8;
+    return guarded([&]() -> int {
+        Geometry g;
+        if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
+        if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+        for (int sign = 0; sign < 2; ++sign) {
+            const uint16_t *l = sign ? neg : pos;
+            for (int c = 0; c < N; ++c)
+                for (int i = 1; i < g.half; ++i) {
+                    if (i % g.n_lane == 0) continue;  // run start: absolute
+                    size_t o = (size_t)c * g.half + i;
+                    if (l[o] <= l[o - 1]) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending");
+                    if (l[o] - l[o - 1] > 127) return 16;
+                }
+        }
+        return 8;
+    });
 }
 
 size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits)
@@ -625,15 +644,19 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
 
 int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out)
 {
-    if (pos && neg)
-        for (size_t i = 0, n = (size_t)N * (S / 2); i < n; ++i)
-            if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
-    return delta_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k, bits);
+    return guarded([&]() -> int {
+        if (pos && neg)
+            for (size_t i = 0, n = (size_t)N * (S / 2); i < n; ++i)
+                if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
+        return delta_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k, bits);
+    });
 }
 
 int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg)
 {
-    return delta_walk(false, (void *)packed, pos, neg, K, N, S, split_k, bits);
+    return guarded([&]() -> int {
+        return delta_walk(false, (void *)packed, pos, neg, K, N, S, split_k, bits);
+    });
 }
 
 // ------------------------------------------------------------------------ i2s
@@ -665,36 +688,40 @@ static inline size_t i2s_word_index(int Kp, int c, int g16)
 
 int sptmm_pack_i2s(const int8_t *W, int K, int N, void *out)
 {
-    if (K <= 0 || N <= 0 || K % 16 || N % 16) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
-    if (!W || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const int Kp = i2s_padded_k(K);
-    uint32_t *o = (uint32_t *)out;
-    std::vector<int> bad(N, 0);
-    parallel_columns(N, [&](int c) {
-        for (int g16 = 0; g16 < Kp / 16; ++g16) {
-            int8_t w16[16] = {0};
-            if (g16 * 16 < K) {
-                memcpy(w16, W + (size_t)c * K + 16 * g16, 16);
-                for (int e = 0; e < 16; ++e)
-                    if (w16[e] < -1 || w16[e] > 1) bad[c] = 1;
+    return guarded([&]() -> int {
+        if (K <= 0 || N <= 0 || K % 16 || N % 16) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
+        if (!W || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        const int Kp = i2s_padded_k(K);
+        uint32_t *o = (uint32_t *)out;
+        std::vector<int> bad(N, 0);
+        parallel_columns(N, [&](int c) {
+            for (int g16 = 0; g16 < Kp / 16; ++g16) {
+                int8_t w16[16] = {0};
+                if (g16 * 16 < K) {
+                    memcpy(w16, W + (size_t)c * K + 16 * g16, 16);
+                    for (int e = 0; e < 16; ++e)
+                        if (w16[e] < -1 || w16[e] > 1) bad[c] = 1;
+                }
+                o[i2s_word_index(Kp, c, g16)] = sptmm_i2s_pack_word(w16);
             }
-            o[i2s_word_index(Kp, c, g16)] = sptmm_i2s_pack_word(w16);
-        }
+        });
+        for (int c = 0; c < N; ++c)
+            if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d holds a weight outside {-1,0,1}", c);
+        return SPTMM_OK;
     });
-    for (int c = 0; c < N; ++c)
-        if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d holds a weight outside {-1,0,1}", c);
-    return SPTMM_OK;
 }
 
 int sptmm_unpack_i2s(const void *packed, int K, int N, int8_t *W)
 {
-    if (K <= 0 || N <= 0 || K % 16 || N % 16) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
-    if (!W || !packed) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const int Kp = i2s_padded_k(K);
-    const uint32_t *p = (const uint32_t *)packed;
-    for (int c = 0; c < N; ++c)
-        for (int g16 = 0; g16 < K / 16; ++g16) sptmm_i2s_decode_word(p[i2s_word_index(Kp, c, g16)], W + (size_t)c * K + 16 * g16);
-    return SPTMM_OK;
+    return guarded([&]() -> int {
+        if (K <= 0 || N <= 0 || K % 16 || N % 16) return fail(SPTMM_ERR_INVALID, "K and N must be positive multiples of 16");
+        if (!W || !packed) return fail(SPTMM_ERR_INVALID, "null pointer");
+        const int Kp = i2s_padded_k(K);
+        const uint32_t *p = (const uint32_t *)packed;
+        for (int c = 0; c < N; ++c)
+            for (int g16 = 0; g16 < K / 16; ++g16) sptmm_i2s_decode_word(p[i2s_word_index(Kp, c, g16)], W + (size_t)c * K + 16 * g16);
+        return SPTMM_OK;
+    });
 }
 
 }  // extern "C"

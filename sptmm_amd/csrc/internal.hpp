@@ -4,6 +4,8 @@
 #include <cstdarg>
 #include <cstddef>
 #include <cstdint>
+#include <exception>
+#include <new>
 #include <vector>
 
 #include "../../include/sptmm.h"
@@ -11,6 +13,18 @@
 namespace sptmm {
 
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Body of an entry point that allocates on the host: no C++ exception may cross the C ABI.
+template <class F> int guarded(F body) noexcept
+{
+    try {
+        return body();
+    } catch (const std::bad_alloc &) {
+        return fail(SPTMM_ERR_NOMEM, "out of host memory");
+    } catch (const std::exception &e) {
+        return fail(SPTMM_ERR_INVALID, "%s", e.what());
+    }
+}
 
 // ---- geometry of the wave64 streams --------------------------------------
 // One "task" is the work of one 64-lane wavefront: G = 64/L columns, L lanes

@@ -14,6 +14,7 @@
 // activation tile keeps behind row K-1.  stride = header + 128 * entry_bytes * n_max.
 #include <algorithm>
 #include <cstring>
+#include <exception>
 #include <thread>
 #include <vector>
 
@@ -26,16 +27,24 @@ namespace {
 template <class F>
 void parallel_for(int n, F f)
 {
+    // worker threads; the first exception any of them meets is rethrown on the calling thread
     unsigned hw = std::thread::hardware_concurrency();
     int nt = (int)std::min<unsigned>(hw ? hw : 1, 16);
     if (n < 64) nt = 1;
     std::vector<std::thread> th;
+    std::vector<std::exception_ptr> err(nt);
     for (int t = 0; t < nt; ++t)
-        th.emplace_back([=] {
-            int i0 = (int)((long)n * t / nt), i1 = (int)((long)n * (t + 1) / nt);
-            for (int i = i0; i < i1; ++i) f(i);
+        th.emplace_back([=, &err] {
+            try {
+                int i0 = (int)((long)n * t / nt), i1 = (int)((long)n * (t + 1) / nt);
+                for (int i = i0; i < i1; ++i) f(i);
+            } catch (...) {
+                err[t] = std::current_exception();
+            }
         });
     for (auto &t : th) t.join();
+    for (auto &e : err)
+        if (e) std::rethrow_exception(e);
 }
 
 struct RaggedPlan {
@@ -249,37 +258,41 @@ extern "C" {
 
 int sptmm_generate_ternary_iid(int K, int N, uint32_t seed, double p_pos, double p_neg, int8_t *W)
 {
-    if (int rc = check_ragged_shape(K, N)) return rc;
-    if (!W) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (!(p_pos >= 0.0) || !(p_neg >= 0.0) || p_pos + p_neg > 1.0) return fail(SPTMM_ERR_INVALID, "probabilities must be >= 0 and sum to at most 1");
-    const uint32_t t_pos = (uint32_t)(p_pos * 16777216.0), t_neg = (uint32_t)((p_pos + p_neg) * 16777216.0);
-    parallel_for(N, [&](int c) {
-        uint32_t st = seed ^ (0x9E3779B9u * (uint32_t)(c + 1));
-        if (!st) st = 1u;
-        int8_t *w = W + (size_t)c * K;
-        for (int r = 0; r < K; ++r) {
-            st ^= st << 13;
-            st ^= st >> 17;
-            st ^= st << 5;
-            const uint32_t u = st >> 8;
-            w[r] = u < t_pos ? (int8_t)1 : (u < t_neg ? (int8_t)-1 : (int8_t)0);
-        }
+    return guarded([&]() -> int {
+        if (int rc = check_ragged_shape(K, N)) return rc;
+        if (!W) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (!(p_pos >= 0.0) || !(p_neg >= 0.0) || p_pos + p_neg > 1.0) return fail(SPTMM_ERR_INVALID, "probabilities must be >= 0 and sum to at most 1");
+        const uint32_t t_pos = (uint32_t)(p_pos * 16777216.0), t_neg = (uint32_t)((p_pos + p_neg) * 16777216.0);
+        parallel_for(N, [&](int c) {
+            uint32_t st = seed ^ (0x9E3779B9u * (uint32_t)(c + 1));
+            if (!st) st = 1u;
+            int8_t *w = W + (size_t)c * K;
+            for (int r = 0; r < K; ++r) {
+                st ^= st << 13;
+                st ^= st >> 17;
+                st ^= st << 5;
+                const uint32_t u = st >> 8;
+                w[r] = u < t_pos ? (int8_t)1 : (u < t_neg ? (int8_t)-1 : (int8_t)0);
+            }
+        });
+        return SPTMM_OK;
     });
-    return SPTMM_OK;
 }
 
 int sptmm_dense_from_i2s_words(const uint32_t *words, int K, int N, int8_t *W)
 {
-    if (K <= 0 || N <= 0 || K % 16) return fail(SPTMM_ERR_INVALID, "K must be a positive multiple of 16");
-    if (!words || !W) return fail(SPTMM_ERR_INVALID, "null pointer");
-    for (int c = 0; c < N; ++c)
-        for (int g16 = 0; g16 < K / 16; ++g16) {
-            int8_t *w = W + (size_t)c * K + 16 * g16;
-            sptmm_i2s_decode_word(words[(size_t)c * (K / 16) + g16], w);
-            for (int e = 0; e < 16; ++e)
-                if (w[e] < -1 || w[e] > 1) return fail(SPTMM_ERR_INVALID, "column %d, row %d: code 0 is not a ternary weight", c, 16 * g16 + e);
-        }
-    return SPTMM_OK;
+    return guarded([&]() -> int {
+        if (K <= 0 || N <= 0 || K % 16) return fail(SPTMM_ERR_INVALID, "K must be a positive multiple of 16");
+        if (!words || !W) return fail(SPTMM_ERR_INVALID, "null pointer");
+        for (int c = 0; c < N; ++c)
+            for (int g16 = 0; g16 < K / 16; ++g16) {
+                int8_t *w = W + (size_t)c * K + 16 * g16;
+                sptmm_i2s_decode_word(words[(size_t)c * (K / 16) + g16], w);
+                for (int e = 0; e < 16; ++e)
+                    if (w[e] < -1 || w[e] > 1) return fail(SPTMM_ERR_INVALID, "column %d, row %d: code 0 is not a ternary weight", c, 16 * g16 + e);
+            }
+        return SPTMM_OK;
+    });
 }
 
 size_t sptmm_pack_ragged_bytes(const int8_t *W, int K, int N, int kind, int split_k, int *bits, size_t *read_bytes, int *n_min,
@@ -297,68 +310,72 @@ size_t sptmm_pack_ragged_bytes(const int8_t *W, int K, int N, int kind, int spli
 
 int sptmm_pack_ragged(const int8_t *W, int K, int N, int kind, int split_k, int bits, void *out)
 {
-    RaggedPlan pl;
-    if (int rc = ragged_plan(W, K, N, kind, split_k, bits, &pl)) return rc;
-    if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
-    memset(out, 0, pl.counts_bytes + pl.stride * pl.g.tasks);
-    if (kind == SPTMM_KIND_U16)
-        pack_u16(pl, (uint8_t *)out);
-    else
-        pack_gaps(pl, (uint8_t *)out);
-    return SPTMM_OK;
+    return guarded([&]() -> int {
+        RaggedPlan pl;
+        if (int rc = ragged_plan(W, K, N, kind, split_k, bits, &pl)) return rc;
+        if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        memset(out, 0, pl.counts_bytes + pl.stride * pl.g.tasks);
+        if (kind == SPTMM_KIND_U16)
+            pack_u16(pl, (uint8_t *)out);
+        else
+            pack_gaps(pl, (uint8_t *)out);
+        return SPTMM_OK;
+    });
 }
 
 int sptmm_unpack_ragged(const void *packed, int K, int N, int kind, int split_k, int bits, int8_t *W)
 {
-    if (int rc = check_ragged_shape(K, N)) return rc;
-    if (kind != SPTMM_KIND_U16 && kind != SPTMM_KIND_DELTA) return fail(SPTMM_ERR_INVALID, "ragged streams are u16 lists or gap streams");
-    Geometry g;
-    if (int rc = make_ragged_geometry(N, split_k, kind == SPTMM_KIND_U16 ? 256 : 64, &g)) return rc;
-    if (!packed || !W) return fail(SPTMM_ERR_INVALID, "null pointer");
-    const bool gaps = kind == SPTMM_KIND_DELTA;
-    if (gaps ? (bits != 8 && bits != 16) : bits != 0) return fail(SPTMM_ERR_INVALID, "delta bits must be 8 or 16 (0 for u16 lists)");
-    const int esz = gaps ? bits / 8 : 2, hdr = gaps ? 256 : 0, sh = gaps ? 0 : ragged_index_shift(K);
-    const uint32_t *pre = (const uint32_t *)packed;
-    const uint32_t n_max = pre[2];
-    if (pre[0] != RAGGED_MAGIC || pre[1] != (uint32_t)g.tasks || n_max < 1 || n_max > 65535 || pre[3] < 1 || pre[3] > n_max)
-        return fail(SPTMM_ERR_INVALID, "not a ragged stream of this shape");
-    const uint16_t *counts = (const uint16_t *)((const uint8_t *)packed + 16);
-    const uint8_t *base = (const uint8_t *)packed + ragged_counts_bytes(g.tasks);
-    const size_t stride = hdr + (size_t)128 * esz * n_max;
-    memset(W, 0, (size_t)K * N);
-    std::vector<int> bad(g.tasks, 0);
-    parallel_for(N / g.G, [&](int ci) {  // all tasks of the columns ci*G .. ci*G+G-1
-        for (int part = 0; part < g.W; ++part) {
-            const int task = ci * g.W + part;
-            const uint8_t *t = base + (size_t)task * stride;
-            const uint32_t n = counts[task];
-            if (n < pre[3] || n > n_max) {
-                bad[task] = 1;
-                continue;
-            }
-            for (int sign = 0; sign < 2; ++sign)
-                for (int lane = 0; lane < 64; ++lane) {
-                    const int col = g.W > 1 ? ci : ci * g.G + lane / g.L;
-                    int row = gaps ? *(const uint16_t *)(t + sign * 128 + lane * 2) : 0;
-                    for (int i = 0; i < (int)n; ++i) {
-                        const uint8_t *cell = t + hdr + slot_offset((int)n, esz, sign, lane, i);
-                        const int f = esz == 1 ? (gaps ? (int)(int8_t)*cell : (int)*cell) : (int)*(const uint16_t *)cell;
-                        row = gaps ? row + f : f >> sh;
-                        if (row < 0 || row >= K + 64) {
-                            bad[task] = 1;
-                            continue;
-                        }
-                        if (row >= K) continue;  // padding
-                        int8_t &w = W[(size_t)col * K + row];
-                        if (w) bad[task] = 1;  // a row may appear once per column
-                        w = sign ? (int8_t)-1 : (int8_t)1;
-                    }
+    return guarded([&]() -> int {
+        if (int rc = check_ragged_shape(K, N)) return rc;
+        if (kind != SPTMM_KIND_U16 && kind != SPTMM_KIND_DELTA) return fail(SPTMM_ERR_INVALID, "ragged streams are u16 lists or gap streams");
+        Geometry g;
+        if (int rc = make_ragged_geometry(N, split_k, kind == SPTMM_KIND_U16 ? 256 : 64, &g)) return rc;
+        if (!packed || !W) return fail(SPTMM_ERR_INVALID, "null pointer");
+        const bool gaps = kind == SPTMM_KIND_DELTA;
+        if (gaps ? (bits != 8 && bits != 16) : bits != 0) return fail(SPTMM_ERR_INVALID, "delta bits must be 8 or 16 (0 for u16 lists)");
+        const int esz = gaps ? bits / 8 : 2, hdr = gaps ? 256 : 0, sh = gaps ? 0 : ragged_index_shift(K);
+        const uint32_t *pre = (const uint32_t *)packed;
+        const uint32_t n_max = pre[2];
+        if (pre[0] != RAGGED_MAGIC || pre[1] != (uint32_t)g.tasks || n_max < 1 || n_max > 65535 || pre[3] < 1 || pre[3] > n_max)
+            return fail(SPTMM_ERR_INVALID, "not a ragged stream of this shape");
+        const uint16_t *counts = (const uint16_t *)((const uint8_t *)packed + 16);
+        const uint8_t *base = (const uint8_t *)packed + ragged_counts_bytes(g.tasks);
+        const size_t stride = hdr + (size_t)128 * esz * n_max;
+        memset(W, 0, (size_t)K * N);
+        std::vector<int> bad(g.tasks, 0);
+        parallel_for(N / g.G, [&](int ci) {  // all tasks of the columns ci*G .. ci*G+G-1
+            for (int part = 0; part < g.W; ++part) {
+                const int task = ci * g.W + part;
+                const uint8_t *t = base + (size_t)task * stride;
+                const uint32_t n = counts[task];
+                if (n < pre[3] || n > n_max) {
+                    bad[task] = 1;
+                    continue;
                 }
-        }
+                for (int sign = 0; sign < 2; ++sign)
+                    for (int lane = 0; lane < 64; ++lane) {
+                        const int col = g.W > 1 ? ci : ci * g.G + lane / g.L;
+                        int row = gaps ? *(const uint16_t *)(t + sign * 128 + lane * 2) : 0;
+                        for (int i = 0; i < (int)n; ++i) {
+                            const uint8_t *cell = t + hdr + slot_offset((int)n, esz, sign, lane, i);
+                            const int f = esz == 1 ? (gaps ? (int)(int8_t)*cell : (int)*cell) : (int)*(const uint16_t *)cell;
+                            row = gaps ? row + f : f >> sh;
+                            if (row < 0 || row >= K + 64) {
+                                bad[task] = 1;
+                                continue;
+                            }
+                            if (row >= K) continue;  // padding
+                            int8_t &w = W[(size_t)col * K + row];
+                            if (w) bad[task] = 1;  // a row may appear once per column
+                            w = sign ? (int8_t)-1 : (int8_t)1;
+                        }
+                    }
+            }
+        });
+        for (int t = 0; t < g.tasks; ++t)
+            if (bad[t]) return fail(SPTMM_ERR_INVALID, "corrupt ragged stream (task %d)", t);
+        return SPTMM_OK;
     });
-    for (int t = 0; t < g.tasks; ++t)
-        if (bad[t]) return fail(SPTMM_ERR_INVALID, "corrupt ragged stream (task %d)", t);
-    return SPTMM_OK;
 }
 
 }  // extern "C"
