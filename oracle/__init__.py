@@ -188,3 +188,29 @@ def make_x_normal(seed: int, M: int, K: int, dtype=np.float16) -> np.ndarray:
     """~N(0,1) activations, seeded, rounded to `dtype`."""
     rng = np.random.default_rng(seed)
     return rng.standard_normal((M, K)).astype(dtype)
+
+
+# ---- the wrapper BitNet inference puts around the integer GEMV (no reference code: the reference
+# ---- only passes an unused scale, main.cu:1862).  Every step is one correctly rounded float32
+# ---- operation, so an implementation that follows the same order matches bit for bit.
+def bf16_bits(x32: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit patterns (round to nearest even), as uint16."""
+    b = np.ascontiguousarray(x32, np.float32).view(np.uint32)
+    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def quantise_rows(xf: np.ndarray):
+    """Per row: a = max(max|x|, 1e-5), s = 127 / a, q = clip(rint(x * s), -127, 127) (round-half-even).
+    -> (q int8 [M][K], a float32 [M])."""
+    xf = xf.astype(np.float32)
+    a = np.maximum(np.abs(xf).max(axis=1), np.float32(1e-5)).astype(np.float32)
+    s = (np.float32(127.0) / a).astype(np.float32)
+    q = np.clip(np.rint(xf * s[:, None]), -127, 127).astype(np.int8)
+    return q, a
+
+
+def rescale(C: np.ndarray, a: np.ndarray, w_scale: float) -> np.ndarray:
+    """y = float32(C) * (a / 127) * w_scale, evaluated in this order in float32."""
+    inv = (a / np.float32(127.0)).astype(np.float32)
+    return ((C.astype(np.float32) * inv[:, None]).astype(np.float32) * np.float32(w_scale)).astype(np.float32)
+

@@ -1,6 +1,7 @@
 """GPU parity of the fused quantise -> GEMV -> rescale entry point (sptmm_gemv_q8).
 
-Reference arithmetic, restated in numpy float32 exactly as include/sptmm.h states it:
+Reference arithmetic, restated in numpy float32 (oracle.quantise_rows / oracle.rescale) exactly as
+include/sptmm.h states it:
     a_m = max(max_k |x[m][k]|, 1e-5);  s_m = 127 / a_m;  q = clip(rint(x * s_m), -127, 127)   (round-half-even)
     C = q . W  (exact int32: the CPU oracle's sums);  y = float(C) * (a_m / 127) * w_scale
 Every step is a single correctly rounded float32 operation, so the result must match bit for bit; the
@@ -22,23 +23,7 @@ def device():
     return sp.device_init(0)
 
 
-def bf16_bits(x32: np.ndarray) -> np.ndarray:
-    """float32 -> bf16 bit patterns (round to nearest even), as uint16."""
-    b = x32.astype(np.float32).view(np.uint32)
-    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
-
-
-def quantise_ref(xf: np.ndarray):
-    xf = xf.astype(np.float32)
-    a = np.maximum(np.abs(xf).max(axis=1), np.float32(1e-5)).astype(np.float32)
-    s = (np.float32(127.0) / a).astype(np.float32)
-    q = np.clip(np.rint(xf * s[:, None]), -127, 127).astype(np.int8)
-    return q, a
-
-
-def y_ref(C: np.ndarray, a: np.ndarray, w_scale: float) -> np.ndarray:
-    inv = (a / np.float32(127.0)).astype(np.float32)
-    return ((C.astype(np.float32) * inv[:, None]).astype(np.float32) * np.float32(w_scale)).astype(np.float32)
+bf16_bits, quantise_ref, y_ref = oracle.bf16_bits, oracle.quantise_rows, oracle.rescale
 
 
 def rows(seed, M, K, dtype):

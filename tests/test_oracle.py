@@ -189,3 +189,21 @@ def test_f64_reference_matches_dense():
     X = oracle.make_x_normal(3, 2, K, np.float16)
     want = X.astype(np.float64) @ W.T.astype(np.float64)
     assert np.allclose(oracle.sptmm_f64(X, pos, neg), want, rtol=0, atol=1e-9)
+
+
+def test_quantise_and_rescale_known_answers():
+    # s = 1 exactly when the row maximum is 127: q = rint(x), ties to even
+    x = np.array([[0.5, 1.5, 2.5, -0.5, -1.5, 3.49, -3.51, 127.0]], np.float32)
+    q, a = oracle.quantise_rows(x)
+    assert a.tolist() == [127.0] and q.tolist() == [[0, 2, 2, 0, -2, 3, -4, 127]]
+    # a row of zeros: the scale clamps at 1e-5, every q is 0
+    q, a = oracle.quantise_rows(np.zeros((1, 4), np.float32))
+    assert q.tolist() == [[0, 0, 0, 0]] and a[0] == np.float32(1e-5)
+    # maximum 2: s = 63.5, 1.0 -> 63.5 -> 64 (tie to even), -2 -> -127
+    q, a = oracle.quantise_rows(np.array([[1.0, -2.0, 0.0078125]], np.float32))
+    assert q.tolist() == [[64, -127, 0]]
+    y = oracle.rescale(np.array([[254, -127]]), np.array([127.0], np.float32), 0.5)
+    assert y.tolist() == [[127.0, -63.5]]
+    # bf16: 1 + 2^-8 is a tie between 1.0 and 1 + 2^-7 -> even (0x3f80); 1 + 3*2^-8 rounds up to 1 + 2^-6
+    bits = oracle.bf16_bits(np.array([1.0, 1.00390625, 1.01171875, -2.5], np.float32))
+    assert [hex(b) for b in bits] == ["0x3f80", "0x3f80", "0x3f82", "0xc020"]
