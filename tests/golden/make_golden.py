@@ -62,6 +62,20 @@ def make_x(seed, M, K):
     return out.reshape(M, K)
 
 
+def generate_iid(K, N, seed, p_pos, p_neg):
+    """Independent entries: per column a xorshift32 stream seeded seed ^ 0x9E3779B9*(col+1) (0 -> 1);
+    entry = top 24 bits of the next state: below p_pos*2^24 -> +1, below (p_pos+p_neg)*2^24 -> -1."""
+    state = (np.uint32(seed) ^ (np.uint32(0x9E3779B9) * np.arange(1, N + 1, dtype=np.uint32))).astype(np.uint32)
+    state[state == 0] = 1
+    t_pos, t_neg = np.uint32(int(p_pos * 16777216.0)), np.uint32(int((p_pos + p_neg) * 16777216.0))
+    W = np.zeros((N, K), np.int8)
+    for r in range(K):
+        state = xorshift32_vec(state)
+        u = state >> np.uint32(8)
+        W[:, r] = np.where(u < t_pos, 1, np.where(u < t_neg, -1, 0))
+    return W
+
+
 def sha(a):
     return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
 
@@ -97,6 +111,15 @@ def main():
                                      "sha256_C": sha(Cm), "C_head": Cm[0, :8].tolist()})
         out["matrices"].append(entry)
         print(K, N, S, entry["sha256_W_colmajor"][:16])
+    out["iid_matrices"] = []
+    for K, N, seed, pp, pn in ((256, 16, 1, 0.3, 0.3), (2560, 640, 0xABCD, 0.35, 0.25), (6912, 2560, 0x2B, 0.3, 0.3)):
+        W = generate_iid(K, N, seed, pp, pn)
+        X = make_x(0xC0FFEE ^ 4, 4, K)
+        Cm = (X.astype(np.int64) @ W.T.astype(np.int64)).astype(np.int32)
+        out["iid_matrices"].append({"K": K, "N": N, "seed": seed, "p_pos": pp, "p_neg": pn, "sha256_W_colmajor": sha(W),
+                                    "nnz": int((W != 0).sum()), "x_seed": 0xC0FFEE ^ 4, "M": 4, "sha256_C": sha(Cm),
+                                    "C_head": Cm[0, :8].tolist()})
+        print("iid", K, N, out["iid_matrices"][-1]["sha256_W_colmajor"][:16])
     with open(os.path.join(HERE, "generator_kats.json"), "w") as f:
         json.dump(out, f, indent=1)
 

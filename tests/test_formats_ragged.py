@@ -215,3 +215,15 @@ def test_argument_errors():
     assert inf["nnz"] == 0 and inf["n_max"] == 1 and (sp.unpack_ragged(packed, 64, 16, U16, 32) == 0).all()
     with pytest.raises(sp.SptmmError):
         sp.unpack_ragged(np.zeros(4096, np.uint8), 64, 16, U16, 32)  # no preamble
+
+
+def test_iid_generator_matches_golden_fixture(golden_dir):
+    import hashlib
+    import json
+    import os
+
+    kats = json.load(open(os.path.join(golden_dir, "generator_kats.json")))["iid_matrices"]
+    assert len(kats) >= 3
+    for e in kats:
+        W = sp.generate_ternary_iid(e["K"], e["N"], e["seed"], e["p_pos"], e["p_neg"])
+        assert hashlib.sha256(W.tobytes()).hexdigest() == e["sha256_W_colmajor"] and int((W != 0).sum()) == e["nnz"]
