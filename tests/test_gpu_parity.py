@@ -329,6 +329,23 @@ def test_argument_errors_are_status_codes():
         o.free()
 
 
+def test_tile_limit_and_largest_k():
+    """One activation row takes 4 bytes of LDS per row of K: K = 40,880 is the last that fits 160 KB."""
+    for K, fits in ((40880, True), (40896 + 64, False)):
+        N, S = 32, 512
+        _, pos, neg = sp.generate_ternary(K, N, S)
+        X = x_i8(K, 1, K)
+        say("tile limit K", K)
+        for w in (sp.Weights.upload_u16(pos, neg, K, 32), sp.Weights.upload_delta(pos, neg, K, 32)):
+            if fits:
+                assert (w.matmul(X) == oracle.sptmm_i8(X, pos, neg)).all()
+            else:
+                with pytest.raises(sp.SptmmError) as e:
+                    w.matmul(X)
+                assert e.value.code == -2 and "LDS" in str(e.value)
+            w.free()
+
+
 def test_streams_and_clone():
     K, N, S = 2560, 640, 1536
     _, pos, neg = matrix(K, N, S)
