@@ -292,6 +292,18 @@ int main(int argc, char **argv)
                 CHECK_SPTMM(sptmm_measure_gemv(cc.data(), (int)cc.size(), a, x_d, M, c_d, iters, 0, stream, &us_cold));
                 printf(" cold[%d copies]=%.3f (%.1f GB/s, %.1f%%)", (int)cc.size(), us_cold, bytes / us_cold / 1e3,
                        bytes / us_cold / 1e3 / dev.peak_hbm_gbps * 100.0);
+                if (a == 0) {
+                    // the same copies, up to 32 GEMVs per launch (sptmm_gemv_i8_batched)
+                    const int nb = (int)std::min<size_t>(cc.size(), 32);
+                    void *cb = nullptr;
+                    double us_bat = 0;
+                    CHECK_SPTMM(sptmm_malloc(&cb, sizeof(int) * (size_t)M * N * nb));
+                    CHECK_SPTMM(sptmm_measure_gemv(cc.data(), nb, 0, x_d, M, cb, 2 * nb, 3, stream, &us_bat));
+                    CHECK_SPTMM(sptmm_measure_gemv(cc.data(), nb, 0, x_d, M, cb, std::max(iters, nb), 3, stream, &us_bat));
+                    CHECK_SPTMM(sptmm_free(cb));
+                    printf(" batched[%d per launch]=%.3f (%.1f GB/s, %.1f%%)", nb, us_bat, bytes / us_bat / 1e3,
+                           bytes / us_bat / 1e3 / dev.peak_hbm_gbps * 100.0);
+                }
                 for (size_t i = 1; i < copies.size(); ++i) sptmm_weights_free(copies[i]);
             }
             printf(" bytes=%.0f kind=%d split_k=%d delta_bits=%d\n", bytes, wi.kind, wi.split_k, wi.delta_bits);
