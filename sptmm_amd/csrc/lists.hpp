@@ -38,9 +38,11 @@ template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 // The running sums of one lane: acc[m] (+|-)= X[m][k] for every gathered row k.
 // int8 activations with MT > 1 keep the tile's bytes biased by 128 (unsigned) and
 // add them four rows at a time into 16-bit fields of plain 32-bit registers --
-// two masks, a shift and two adds per four rows, all in the short VOP2 encoding,
-// against four dot4 instructions (measured on gfx950: a VOP3 instruction costs
-// about twice a VOP2 one).  A field holds at most 257 entries (257 * 255 < 65536);
+// two masks, a shift and two adds per four rows in place of four dot4
+// instructions with one-hot selectors (in an issue-rate probe on gfx950 dot4 and
+// the other VOP3 forms took twice as long as a plain add; on the M=4 headline
+// shape the change was worth 78 % -> 82 % of HBM peak in batched launches).
+// A field holds at most 257 entries (257 * 255 < 65536);
 // flush() widens the fields into acc[] and has to be called at least that often.
 // Both signs of a lane always gather the same number of entries, so the bias cancels.
 template <typename Act, int MT> struct Sums {
@@ -144,8 +146,8 @@ template <int B> __device__ __forceinline__ void add_signed_byte(u32 &run, u32 d
 
 // `run` is the current row of a gap stream: the row index itself with 8-bit gaps,
 // the byte offset of the row's slot in the tile with 16-bit gaps.  fetch() turns
-// the low NBYTES of `d` into tile reads (all of them issued before anything is
-// added up, so a round keeps its 16 or 32 LDS reads in flight together).
+// the low NBYTES of `d` into tile reads; the adds follow separately so that the
+// compiler is free to keep several reads in flight.
 template <typename Act, int MT, int MODE, bool PRE, int NBYTES>
 __device__ __forceinline__ void fetch(const unsigned char *lds, u32 d, u32 &run, typename Sums<Act, MT>::Raw *r)
 {
