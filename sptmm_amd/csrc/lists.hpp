@@ -433,11 +433,13 @@ struct ListsBody {
     // RF > 0: the task has exactly RF full rounds (ragged: RF to RF + XMAX) and
     // all of them live in registers, loaded and consumed in straight-line code
     // (so every wait on the stream is for one round only).  RF == 0: any number
-    // of rounds, through a ring of RING rounds in flight.
+    // of rounds, through a ring of RING rounds in flight.  RF == -1: no full round at all
+    // (ragged: up to XMAX), only the tail.
     template <int RF>
     static __device__ __forceinline__ void run(const ListParams &p, unsigned char *smem)
     {
-        constexpr int NB = RF > 0 ? RF : RING;
+        constexpr int NR = RF > 0 ? RF : 0;               // full rounds of the straight-line body (RF == -1: none, tails only)
+        constexpr int NB = RF > 0 ? RF : RF == 0 ? RING : 1;
         A *part = reinterpret_cast<A *>(smem + (size_t)(p.K + ZROWS) * SLOT);
         const int tid = threadIdx.x, nt = blockDim.x;
         const int lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
@@ -485,7 +487,7 @@ struct ListsBody {
             if constexpr (RF > 0) {
 #pragma unroll
                 for (int i = 0; i < (RF < EARLY ? RF : EARLY); ++i) buf[i] = load_round(wp, i);
-            } else if (R0 > 0) {
+            } else if (RF == 0 && R0 > 0) {
 #pragma unroll
                 for (int i = 0; i < EARLY; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
             }
@@ -587,10 +589,10 @@ struct ListsBody {
             Sums<Act, MT> acc;
             acc.init();
 
-            if constexpr (RF > 0) {
+            if constexpr (RF != 0) {
                 if (it > 0) {
 #pragma unroll
-                    for (int i = 0; i < RF; ++i) buf[i] = load_round(wp, i);
+                    for (int i = 0; i < NR; ++i) buf[i] = load_round(wp, i);
                 }
             } else {
                 // ring of RING rounds, loads clamped to the task's last round so that they stay unconditional
@@ -606,10 +608,10 @@ struct ListsBody {
                 }
             }
             Round xb[XMAX > 0 ? XMAX : 1];
-            if constexpr (RF > 0 && XMAX > 0) {
+            if constexpr (RF != 0 && XMAX > 0) {
 #pragma unroll
                 for (int x = 0; x < XMAX; ++x)
-                    if (RF + x < R) xb[x] = load_round(wp, RF + x);
+                    if (NR + x < R) xb[x] = load_round(wp, NR + x);
             }
             // ragged tail, requested now and eaten last: at most one round each of 8, 4, 2 (and 1) bytes per lane
             uint2 t8p = make_uint2(0, 0), t8q = make_uint2(0, 0);
@@ -664,11 +666,11 @@ struct ListsBody {
                 }
             } else {
 #pragma unroll
-                for (int i = 0; i < RF; ++i) eat(smem, buf[i], runp, runq, acc);
+                for (int i = 0; i < NR; ++i) eat(smem, buf[i], runp, runq, acc);
                 if constexpr (XMAX > 0) {
 #pragma unroll
                     for (int x = 0; x < XMAX; ++x)
-                        if (RF + x < R) eat(smem, xb[x], runp, runq, acc);
+                        if (NR + x < R) eat(smem, xb[x], runp, runq, acc);
                 }
             }
             if (rem) {
@@ -889,20 +891,23 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel launch");
 }
 
-// Straight-line bodies exist for the u16 and 8-bit run streams
-// with 1, 2, 3, 4, 6 or 8 full rounds per task (ragged streams: for the shortest
+// Straight-line bodies exist for tasks
+// with 1, 2, 3, 4, 6 or 8 full rounds (ragged streams: for the shortest
 // task, when the longest has at most XMAX more); everything else takes the ring.
 template <typename Act, int MT, int MODE, bool PRE, bool VAR>
 static int launch_lists_t(const GemvArgs &a, hipStream_t st)
 {
-    if constexpr (MODE < 2) {
-        constexpr int E16 = MODE == 1 ? 16 : 8;
+    {
+        constexpr int E16 = 16 / Flavour<MODE>::ESZ;
         int rf = (VAR ? a.n_min : a.n_lane) / E16;
         if constexpr (VAR) {
             rf = rf >= 8 ? 8 : rf >= 6 ? 6 : rf == 5 ? 4 : rf;
             if (a.n_max / E16 - rf > ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) rf = 0;
         }
         switch (rf) {
+        case 0:
+            if ((VAR ? a.n_max : a.n_lane) / E16 <= ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) return launch_lists_rf<Act, MT, MODE, PRE, VAR, -1>(a, st);
+            break;
         case 1: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 1>(a, st);
         case 2: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 2>(a, st);
         case 3: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 3>(a, st);
