@@ -194,6 +194,10 @@ int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int
  * arrays of device pointers. */
 int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X_dev, int32_t *const *C_dev, int count,
                           int M, void *stream);
+/* The same for any activation type: act 0 int8 (int32 out), 1 fp16 or 2 fp32
+ * (float out; u16 and gap streams only). */
+int sptmm_gemv_batched(const sptmm_weights *const *ws, const void *const *X_dev, void *const *C_dev, int count, int M,
+                       int act, void *stream);
 
 /* Thin device-memory / stream / event helpers so callers need no HIP headers
  * (the cudaMalloc/cudaMemcpy/cudaEvent* calls of main.cu:767-782, 804-815). */

@@ -11,7 +11,7 @@ __all__ = [
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
     "generate_ternary_iid", "dense_from_i2s_words",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
-    "device_sync", "measure_gemv", "gemv_i8_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
+    "device_sync", "measure_gemv", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
 
 KIND_U16, KIND_DELTA, KIND_I2S = 1, 2, 3
@@ -29,7 +29,7 @@ EXPORTS = [
     "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
-    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_i8_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
+    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_i8_batched", "sptmm_gemv_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
@@ -84,6 +84,7 @@ def lib() -> C.CDLL:
         for n in ("sptmm_gemv_i8", "sptmm_gemv_f16", "sptmm_gemv_f32"):
             getattr(L, n).argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.sptmm_gemv_q8.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p]
+        L.sptmm_gemv_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_gemv_i8_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
         L.sptmm_free.argtypes = [C.c_void_p]
@@ -339,14 +340,19 @@ def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuff
     return us.value
 
 
-def gemv_i8_batched(weights, Xs, Cs, M: int, stream: "Stream | None" = None):
-    """One launch for len(weights) GEMVs of one shape: Cs[i] = Xs[i] . weights[i] (device buffers)."""
+def gemv_batched(weights, Xs, Cs, M: int, act: int = 0, stream: "Stream | None" = None):
+    """One launch for len(weights) GEMVs of one shape: Cs[i] = Xs[i] . weights[i] (device buffers).
+    act: 0 int8 -> int32, 1 fp16 -> fp32, 2 fp32 -> fp32."""
     n = len(weights)
     assert len(Xs) == n and len(Cs) == n
     wa = (C.c_void_p * n)(*[w.handle for w in weights])
     xa = (C.c_void_p * n)(*[x.ptr for x in Xs])
     ca = (C.c_void_p * n)(*[c.ptr for c in Cs])
-    _ck(lib().sptmm_gemv_i8_batched(wa, xa, ca, n, M, stream.handle if stream else None))
+    _ck(lib().sptmm_gemv_batched(wa, xa, ca, n, M, act, stream.handle if stream else None))
+
+
+def gemv_i8_batched(weights, Xs, Cs, M: int, stream: "Stream | None" = None):
+    gemv_batched(weights, Xs, Cs, M, 0, stream)
 
 
 def device_sync():

@@ -407,11 +407,12 @@ int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X, int M, int32_t *C, vo
     return gemv_common(w, X, M, C, stream, ACT_I8);
 }
 
-int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X, int32_t *const *C, int count, int M,
-                          void *stream)
+int sptmm_gemv_batched(const sptmm_weights *const *ws, const void *const *X, void *const *C, int count, int M, int act,
+                       void *stream)
 {
     return guarded([&]() -> int {
         if (!ws || !X || !C || count < 1) return fail(SPTMM_ERR_INVALID, "bad argument");
+        if (act < ACT_I8 || act > ACT_F32) return fail(SPTMM_ERR_INVALID, "act must be 0 (int8), 1 (fp16) or 2 (fp32)");
         if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
         std::vector<const void *> wp(count), xp(count);
         std::vector<void *> cp(count);
@@ -426,8 +427,14 @@ int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X
             xp[i] = X[i];
             cp[i] = C[i];
         }
-        return gemv_common(ws[0], X[0], M, C[0], stream, ACT_I8, count, wp.data(), xp.data(), cp.data());
+        return gemv_common(ws[0], X[0], M, C[0], stream, (ActType)act, count, wp.data(), xp.data(), cp.data());
     });
+}
+
+int sptmm_gemv_i8_batched(const sptmm_weights *const *ws, const int8_t *const *X, int32_t *const *C, int count, int M,
+                          void *stream)
+{
+    return sptmm_gemv_batched(ws, (const void *const *)X, (void *const *)C, count, M, ACT_I8, stream);
 }
 
 int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X, int x_type, int M, float w_scale, float *Y, void *stream)
@@ -532,7 +539,7 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
 {
     if (!ws || n_ws < 1 || !X || !C || iters < 1 || !us_per_call) return fail(SPTMM_ERR_INVALID, "bad argument");
     if (act < 0 || act > 4 || mode < 0 || mode > 3) return fail(SPTMM_ERR_INVALID, "bad act or mode");
-    if (mode == 3 && act != ACT_I8) return fail(SPTMM_ERR_UNSUPPORTED, "batched timing takes int8 activations");
+    if (mode == 3 && act > ACT_F32) return fail(SPTMM_ERR_UNSUPPORTED, "batched timing takes int8, fp16 or fp32 activations");
     // act 3 / 4: the quantising GEMV on fp16 / bf16 rows (w_scale 1)
     auto launch = [&](const sptmm_weights *w) {
         return act >= 3 ? sptmm_gemv_q8(w, (const uint16_t *)X, act == 3 ? SPTMM_X_F16 : SPTMM_X_BF16, M, 1.0f, (float *)C, stream)
@@ -575,13 +582,13 @@ int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const 
         *us_per_call = (double)ms * 1000.0 / ((double)reps * n_ws);
     } else if (mode == 3) {
         // one launch per rotation: all n_ws GEMVs in a single batched dispatch, outputs side by side in C
-        std::vector<const int8_t *> xs(n_ws, (const int8_t *)X);
-        std::vector<int32_t *> cs(n_ws);
-        for (int i = 0; i < n_ws; ++i) cs[i] = (int32_t *)C + (size_t)i * M * ws[0]->info.N;
+        std::vector<const void *> xs(n_ws, X);
+        std::vector<void *> cs(n_ws);
+        for (int i = 0; i < n_ws; ++i) cs[i] = (int32_t *)C + (size_t)i * M * ws[0]->info.N;  // 4 bytes per output, int32 or float
         const int reps = (iters + n_ws - 1) / n_ws;
         M_TRY(hipEventRecord(e0, st));
         for (int r = 0; r < reps; ++r) {
-            rc = sptmm_gemv_i8_batched(ws, xs.data(), cs.data(), n_ws, M, st);
+            rc = sptmm_gemv_batched(ws, xs.data(), cs.data(), n_ws, M, act, st);
             if (rc != SPTMM_OK) goto done;
         }
         M_TRY(hipEventRecord(e1, st));

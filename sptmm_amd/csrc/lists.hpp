@@ -846,7 +846,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     if (a.batch) {
-        if constexpr (sizeof(Act) == 1) {
+        {
             auto kern = lists_kernel_batched<Act, MT, MODE, PRE, VAR, RF>;
             static std::atomic<size_t> lds_granted_b{48 * 1024};
             if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_b)) return rc;
@@ -864,8 +864,6 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
                 if (e != hipSuccess) return hip_fail(e, "lists_kernel_batched launch");
             }
             return SPTMM_OK;
-        } else {
-            return fail(SPTMM_ERR_UNSUPPORTED, "batched launches take int8 activations");
         }
     }
     if (a.quant) {

@@ -172,6 +172,7 @@ def float_rows(st, rows):
         xs = ((0, "i8", sp.make_x_i8(1, M, K)), (1, "f16", rng.standard_normal((M, K)).astype(np.float16)),
               (2, "f32", rng.standard_normal((M, K)).astype(np.float32)))
         cb = sp.DeviceBuffer(4 * M * N)
+        cbb = sp.DeviceBuffer(4 * M * N * 32)
         for enc, split in (("delta", 32), ("u16", 32)):
             w = sp.Weights.upload_delta(pos, neg, K, split) if enc == "delta" else sp.Weights.upload_u16(pos, neg, K, split)
             n = copies_for(w.nbytes)
@@ -182,13 +183,19 @@ def float_rows(st, rows):
                 warm = min(sp.measure_gemv(cps[:1], act, xb, M, cb, 2000, 0, st) for _ in range(3))
                 sp.measure_gemv(cps, act, xb, M, cb, 2 * n, 0, st)
                 cold = min(sp.measure_gemv(cps, act, xb, M, cb, 2000, 0, st) for _ in range(3))
+                nb = min(n, 32)
+                sp.measure_gemv(cps[:nb], act, xb, M, cbb, 4 * nb, 3, st)
+                bat = min(sp.measure_gemv(cps[:nb], act, xb, M, cbb, 64 * nb, 3, st) for _ in range(3))
+                nbytes = w.info["stream_bytes"] + M * K * X.itemsize + 4 * M * N
                 xb.free()
-                print("headline M=%d %s/%d %-3s activations: warm %6.2f us  cold %6.2f us" % (M, enc, split, name, warm, cold), flush=True)
-                rows.append({"shape": "headline", "M": M, "enc": "%s/%d" % (enc, split), "act": name,
-                             "warm_us": round(warm, 3), "cold_us": round(cold, 3)})
+                print("headline M=%d %s/%d %-3s activations: warm %6.2f us  cold %6.2f us  %d per launch %6.2f us (%.1f%% of HBM peak)"
+                      % (M, enc, split, name, warm, cold, nb, bat, nbytes / bat / 1e3 / PEAK_GBPS * 100), flush=True)
+                rows.append({"shape": "headline", "M": M, "enc": "%s/%d" % (enc, split), "act": name, "bytes": nbytes,
+                             "warm_us": round(warm, 3), "cold_us": round(cold, 3), "batched_us": round(bat, 3)})
             for c in cps:
                 c.free()
         cb.free()
+        cbb.free()
 
 
 def main(argv):

@@ -395,6 +395,29 @@ def test_batched_launch_equals_single_launches(kind, M, count):
     st.destroy()
 
 
+@pytest.mark.parametrize("kind", ["u16", "delta"])
+@pytest.mark.parametrize("dtype,act", [(np.float16, 1), (np.float32, 2)])
+def test_batched_launch_float_activations(kind, dtype, act):
+    K, N, S = 2560, 640, 1536
+    _, pos, neg = matrix(K, N, S)
+    base = sp.Weights.upload_u16(pos, neg, K, 32) if kind == "u16" else sp.Weights.upload_delta(pos, neg, K, 32)
+    for M, count in ((1, 4), (4, 3)):
+        ws = [base] + [base.clone() for _ in range(count - 1)]
+        Xs = [oracle.make_x_normal(70 + i, M, K, dtype) for i in range(count)]
+        xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
+        cb = [sp.DeviceBuffer(4 * M * N) for _ in range(count)]
+        say("batched float", kind, dtype.__name__, "M", M, "count", count)
+        sp.gemv_batched(ws, xb, cb, M, act)
+        sp.device_sync()
+        for i in range(count):
+            got = cb[i].to_numpy(np.float32, (M, N))
+            check_fp(got, oracle.sptmm_f64(Xs[i], pos, neg), S)
+            assert (got == base.matmul(Xs[i])).all()  # and bit-identical to the single launch
+        for o in ws[1:] + xb + cb:
+            o.free()
+    base.free()
+
+
 def test_batched_launch_rejects_mixed_shapes():
     _, pos, neg = matrix(512, 48, 256)
     a = sp.Weights.upload_u16(pos, neg, 512, 32)
