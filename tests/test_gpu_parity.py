@@ -76,7 +76,7 @@ def test_u16_headline_shape_bit_exact(split, M, golden_dir):
     assert hashlib.sha256(got.tobytes()).hexdigest() == o["sha256_C"]
 
 
-@pytest.mark.parametrize("M", [2, 3, 5, 7, 8, 9, 16])
+@pytest.mark.parametrize("M", [2, 3, 5, 7, 8, 9, 16, 33, 64])
 def test_u16_row_counts(M):
     K, N, S = 6912, 256, 4096
     say("u16 rows", M)
