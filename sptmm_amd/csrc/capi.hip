@@ -247,9 +247,11 @@ int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out)
         if (!w || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
         sptmm_weights *c = new (std::nothrow) sptmm_weights(*w);
         if (!c) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        c->dev = nullptr;
         hipError_t e = hipMalloc(&c->dev, w->bytes);
         if (e == hipSuccess) e = hipMemcpy(c->dev, w->dev, w->bytes, hipMemcpyDeviceToDevice);
         if (e != hipSuccess) {
+            if (c->dev) (void)hipFree(c->dev);
             delete c;
             return hip_fail(e, "clone weight stream");
         }
@@ -534,8 +536,11 @@ int sptmm_event_elapsed_us(void *a, void *b, double *us)
     *us = (double)ms * 1000.0;
     return SPTMM_OK;
 }
-int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters,
-                       int mode, void *stream, double *us_per_call)
+}  // extern "C"
+
+namespace {
+int measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters, int mode,
+                 void *stream, double *us_per_call)
 {
     if (!ws || n_ws < 1 || !X || !C || iters < 1 || !us_per_call) return fail(SPTMM_ERR_INVALID, "bad argument");
     if (act < 0 || act > 4 || mode < 0 || mode > 3) return fail(SPTMM_ERR_INVALID, "bad act or mode");
@@ -616,6 +621,15 @@ done:
     (void)hipStreamSynchronize(st);
     return rc;
 }
+}  // namespace
+
+extern "C" {
+
+int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters,
+                       int mode, void *stream, double *us_per_call)
+{
+    return guarded([&]() -> int { return measure_gemv(ws, n_ws, act, X, M, C, iters, mode, stream, us_per_call); });
+}
 
 int sptmm_read_kernel(const void *src, size_t bytes, size_t stride_bytes, int regions, void *sink, int workgroups, int launches,
                       void *stream, double *us_per_launch)
@@ -626,7 +640,10 @@ int sptmm_read_kernel(const void *src, size_t bytes, size_t stride_bytes, int re
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0, e1;
     HIP_TRY(hipEventCreate(&e0));
-    HIP_TRY(hipEventCreate(&e1));
+    if (hipError_t ce = hipEventCreate(&e1); ce != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return hip_fail(ce, "hipEventCreate");
+    }
     auto region = [&](int i) { return (const uint8_t *)src + (size_t)(i % regions) * stride_bytes; };
     int rc = launch_read(region(0), bytes, sink, workgroups, stream);  // untimed first launch
     hipError_t e = hipEventRecord(e0, st);

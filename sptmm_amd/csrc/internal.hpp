@@ -23,6 +23,8 @@ template <class F> int guarded(F body) noexcept
         return fail(SPTMM_ERR_NOMEM, "out of host memory");
     } catch (const std::exception &e) {
         return fail(SPTMM_ERR_INVALID, "%s", e.what());
+    } catch (...) {
+        return fail(SPTMM_ERR_INVALID, "unexpected exception");
     }
 }
 
