@@ -321,6 +321,10 @@ struct ListParams {
 };
 
 constexpr int LISTS_MAX_WAVES = 8;  // 512 threads: two wavefronts per SIMD, 256 VGPRs each
+// Eight-row tiles do an order of magnitude more arithmetic per stream byte and a large K leaves
+// room for one workgroup per CU only, so that workgroup has to bring the wavefronts that hide
+// the LDS latency itself: 1024 threads, four wavefronts per SIMD, 128 VGPRs each.
+template <int MT, bool QUANT> constexpr int lists_max_waves() { return MT == 8 && !QUANT ? 16 : LISTS_MAX_WAVES; }
 
 // One round of a task's stream: 16 bytes per lane of the +1 list and of the -1 list.
 struct Round {
@@ -746,7 +750,7 @@ struct ListsBody {
 // blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
 // exactly RF full rounds (straight-line body); RF == 0: any length (ring).
 template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool QUANT = false>
-__global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel(ListParams p)
+__global__ void __launch_bounds__((64 * lists_max_waves<MT, QUANT>())) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     ListsBody<Act, MT, MODE, PRE, VAR, QUANT>::template run<RF>(p, smem);
@@ -762,7 +766,7 @@ struct BatchPtrs {
 };
 
 template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
-__global__ void __launch_bounds__(64 * LISTS_MAX_WAVES) lists_kernel_batched(ListParams p, BatchPtrs b)
+__global__ void __launch_bounds__((64 * lists_max_waves<MT, false>())) lists_kernel_batched(ListParams p, BatchPtrs b)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     p.w = b.w[blockIdx.z];
@@ -803,6 +807,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(a.K + 64) * SLOT;
+    const int max_waves = a.quant ? LISTS_MAX_WAVES : lists_max_waves<MT, false>();
     static std::atomic<int> vgprs{0};  // of the single-GEMV kernel of this instantiation
     int regs = vgprs.load(std::memory_order_relaxed);
     if (!regs) {
@@ -819,7 +824,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     double best = 1e30;
     for (int g = 1; g <= (a.batch ? 1 : 3); ++g) {
         if (tune_wgs > 0 && g != tune_wgs) continue;
-        for (int w = a.W; w <= LISTS_MAX_WAVES; w += a.W) {
+        for (int w = a.W; w <= max_waves; w += a.W) {
             if (g > 1 && g * w > 4 * waves_per_simd) continue;  // the register file of the CU's 4 SIMDs
             if (g > 1 && g * (tile + (size_t)w * MT * 4) > (size_t)a.lds_limit) continue;
             const int blocks = (a.tasks + w - 1) / w;
@@ -835,7 +840,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             }
         }
     }
-    if (tune_wpb > 0 && tune_wpb <= LISTS_MAX_WAVES && tune_wpb % a.W == 0) wpb = tune_wpb;
+    if (tune_wpb > 0 && tune_wpb <= max_waves && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
     const int grid_x = blocks < slots ? blocks : slots;
