@@ -321,10 +321,10 @@ struct ListParams {
 };
 
 constexpr int LISTS_MAX_WAVES = 8;  // 512 threads: two wavefronts per SIMD, 256 VGPRs each
-// Eight-row tiles do an order of magnitude more arithmetic per stream byte and a large K leaves
-// room for one workgroup per CU only, so that workgroup has to bring the wavefronts that hide
-// the LDS latency itself: 1024 threads, four wavefronts per SIMD, 128 VGPRs each.
-template <int MT, bool QUANT> constexpr int lists_max_waves() { return MT == 8 && !QUANT ? 16 : LISTS_MAX_WAVES; }
+// Multi-row int8 tiles do several times the arithmetic per stream byte, and a large K leaves
+// room for one workgroup per CU only, so that workgroup has to bring the wavefronts that fill
+// the four SIMDs itself: 1024 threads, four wavefronts per SIMD, 128 VGPRs each.
+template <typename Act, int MT, bool QUANT> constexpr int lists_max_waves() { return sizeof(Act) == 1 && MT >= 4 && !QUANT ? 16 : LISTS_MAX_WAVES; }
 
 // One round of a task's stream: 16 bytes per lane of the +1 list and of the -1 list.
 struct Round {
@@ -750,7 +750,7 @@ struct ListsBody {
 // blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
 // exactly RF full rounds (straight-line body); RF == 0: any length (ring).
 template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool QUANT = false>
-__global__ void __launch_bounds__((64 * lists_max_waves<MT, QUANT>())) lists_kernel(ListParams p)
+__global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, QUANT>())) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     ListsBody<Act, MT, MODE, PRE, VAR, QUANT>::template run<RF>(p, smem);
@@ -766,7 +766,7 @@ struct BatchPtrs {
 };
 
 template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
-__global__ void __launch_bounds__((64 * lists_max_waves<MT, false>())) lists_kernel_batched(ListParams p, BatchPtrs b)
+__global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, false>())) lists_kernel_batched(ListParams p, BatchPtrs b)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     p.w = b.w[blockIdx.z];
@@ -807,7 +807,9 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(a.K + 64) * SLOT;
-    const int max_waves = a.quant ? LISTS_MAX_WAVES : lists_max_waves<MT, false>();
+    // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better
+    const bool roomy = a.batch && 2 * (tile + (size_t)LISTS_MAX_WAVES * MT * 4) <= (size_t)a.lds_limit;
+    const int max_waves = a.quant || roomy ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>();
     static std::atomic<int> vgprs{0};  // of the single-GEMV kernel of this instantiation
     int regs = vgprs.load(std::memory_order_relaxed);
     if (!regs) {
@@ -843,8 +845,15 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     if (tune_wpb > 0 && tune_wpb <= max_waves && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
-    const int grid_x = blocks < slots ? blocks : slots;
-    const int iters = (blocks + grid_x - 1) / grid_x;
+    int grid_x = blocks < slots ? blocks : slots;
+    int iters = (blocks + grid_x - 1) / grid_x;
+    // A batched launch has workgroups enough to fill the chip along blockIdx.z, and every workgroup
+    // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
+    // per GEMV, four-row tiles 2.83 -> 2.76; nothing for the one-row u16 kernel, which waits on HBM only).
+    if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && MT == 1)) {
+        grid_x = (blocks + 1) / 2;
+        iters = 2;
+    }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
                  a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale};
     size_t lds = (size_t)(a.K + 64) * SLOT + (size_t)wpb * MT * sizeof(typename Acc<Act>::type);
