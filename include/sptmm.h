@@ -215,6 +215,20 @@ int sptmm_event_destroy(void *event);
 int sptmm_event_record(void *event, void *stream);
 int sptmm_event_sync(void *event);
 int sptmm_event_elapsed_us(void *start, void *stop, double *us);
+/* Stream capture: the launches issued on `stream` between _begin and _end (any of
+ * the sptmm_gemv_* calls, in any mix) become one executable HIP graph that
+ * _launch replays -- a decoder layer's fixed sequence of projections as one
+ * submission.  The reference issues its kernels one by one with a device
+ * synchronize after each (main.cu:767-782).  Pointers and shapes are frozen at
+ * capture; the contents of X may change between replays.  `stream` must come
+ * from sptmm_stream_create; capture is thread-local, and a failed call between
+ * _begin and _end still has to be followed by _end, which then reports the
+ * failure.  The graph holds kernel launches only (no memset or copy nodes). */
+int sptmm_graph_begin(void *stream);
+int sptmm_graph_end(void *stream, void **graph);
+int sptmm_graph_launch(void *graph, void *stream);
+int sptmm_graph_destroy(void *graph);
+
 /* The timing loop of measureKernel (main.cu:767-782) around `iters` GEMV
  * launches, kept native so that no interpreter sits between launches.  Launch i
  * uses ws[i % n_ws] (several device copies of one matrix defeat the last-level

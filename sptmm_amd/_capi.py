@@ -11,7 +11,7 @@ __all__ = [
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
     "generate_ternary_iid", "dense_from_i2s_words",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
-    "device_sync", "measure_gemv", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
+    "device_sync", "Graph", "measure_gemv", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
 
 KIND_U16, KIND_DELTA, KIND_I2S = 1, 2, 3
@@ -33,6 +33,7 @@ EXPORTS = [
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
+    "sptmm_graph_begin", "sptmm_graph_end", "sptmm_graph_launch", "sptmm_graph_destroy",
 ]
 
 
@@ -103,6 +104,10 @@ def lib() -> C.CDLL:
         for n in ("sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_event_destroy", "sptmm_event_sync"):
             getattr(L, n).argtypes = [C.c_void_p]
         L.sptmm_event_record.argtypes = [C.c_void_p, C.c_void_p]
+        L.sptmm_graph_begin.argtypes = [C.c_void_p]
+        L.sptmm_graph_end.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.sptmm_graph_launch.argtypes = [C.c_void_p, C.c_void_p]
+        L.sptmm_graph_destroy.argtypes = [C.c_void_p]
         L.sptmm_event_elapsed_us.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]
         _LIB = L
     return _LIB
@@ -266,6 +271,13 @@ class DeviceBuffer:
             _ck(lib().sptmm_memcpy_h2d(b.ptr, _p(a), a.nbytes))
         return b
 
+    def upload(self, a: np.ndarray):
+        """Overwrite the start of the buffer with `a` (synchronous copy)."""
+        a = np.ascontiguousarray(a)
+        assert a.nbytes <= self.nbytes
+        if a.nbytes:
+            _ck(lib().sptmm_memcpy_h2d(self.ptr, _p(a), a.nbytes))
+
     def to_numpy(self, dtype, shape) -> np.ndarray:
         out = np.empty(shape, dtype)
         assert out.nbytes <= self.nbytes
@@ -299,6 +311,39 @@ class Stream:
     def destroy(self):
         if self.handle:
             lib().sptmm_stream_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+
+class Graph:
+    """The launches issued on `stream` inside the `with` block, as one executable HIP graph.
+
+        with sp.Graph(st) as g:
+            w0.gemv_i8(x0, 1, c0, st); w1.gemv_i8(x1, 1, c1, st)
+        g.launch(st)
+    """
+
+    def __init__(self, stream: Stream):
+        self.stream = stream
+        self.handle = C.c_void_p()
+
+    def __enter__(self):
+        _ck(lib().sptmm_graph_begin(self.stream.handle))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = lib().sptmm_graph_end(self.stream.handle, C.byref(self.handle))
+        if exc_type is None:
+            _ck(rc)
+        elif rc == 0:
+            self.destroy()  # the block failed: the capture is closed and its graph dropped
+        return False
+
+    def launch(self, stream: Stream | None = None):
+        _ck(lib().sptmm_graph_launch(self.handle, (stream or self.stream).handle))
+
+    def destroy(self):
+        if self.handle:
+            lib().sptmm_graph_destroy(self.handle)
             self.handle = C.c_void_p()
 
 

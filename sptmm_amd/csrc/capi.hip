@@ -536,6 +536,55 @@ int sptmm_event_elapsed_us(void *a, void *b, double *us)
     *us = (double)ms * 1000.0;
     return SPTMM_OK;
 }
+struct sptmm_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+int sptmm_graph_begin(void *stream)
+{
+    if (!stream) return fail(SPTMM_ERR_INVALID, "capture needs a stream made by sptmm_stream_create");
+    HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return SPTMM_OK;
+}
+
+int sptmm_graph_end(void *stream, void **graph)
+{
+    return guarded([&]() -> int {
+        if (!stream || !graph) return fail(SPTMM_ERR_INVALID, "null pointer");
+        sptmm_graph *g = new (std::nothrow) sptmm_graph();
+        if (!g) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        hipError_t e = hipStreamEndCapture((hipStream_t)stream, &g->graph);
+        if (e == hipSuccess && !g->graph) e = hipErrorStreamCaptureInvalidated;
+        if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) {
+            if (g->graph) (void)hipGraphDestroy(g->graph);
+            delete g;
+            return hip_fail(e, "ending the capture");
+        }
+        *graph = g;
+        return SPTMM_OK;
+    });
+}
+
+int sptmm_graph_launch(void *graph, void *stream)
+{
+    if (!graph) return fail(SPTMM_ERR_INVALID, "null pointer");
+    HIP_TRY(hipGraphLaunch(((sptmm_graph *)graph)->exec, (hipStream_t)stream));
+    return SPTMM_OK;
+}
+
+int sptmm_graph_destroy(void *graph)
+{
+    if (!graph) return SPTMM_OK;
+    sptmm_graph *g = (sptmm_graph *)graph;
+    hipError_t e1 = hipGraphExecDestroy(g->exec), e2 = hipGraphDestroy(g->graph);
+    delete g;
+    if (e1 != hipSuccess) return hip_fail(e1, "hipGraphExecDestroy");
+    if (e2 != hipSuccess) return hip_fail(e2, "hipGraphDestroy");
+    return SPTMM_OK;
+}
+
 }  // extern "C"
 
 namespace {
