@@ -37,20 +37,21 @@ template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 
 // The running sums of one lane: acc[m] (+|-)= X[m][k] for every gathered row k.
 // int8 activations with MT > 1 keep the tile's bytes biased by 128 (unsigned) and
-// add them four rows at a time into 16-bit fields of plain 32-bit registers --
-// two masks, a shift and two adds per four rows in place of four dot4
+// add them four rows at a time into plain 32-bit registers: bytes 0 and 2 masked
+// into two 16-bit fields, and the whole dword shifted right by 8, whose running sum
+// sum(b1) + 2^8 sum(b2) + 2^16 sum(b3) (mod 2^32) separates again once sum(b2) is
+// known -- a mask, a shift and two adds per four rows in place of four dot4
 // instructions with one-hot selectors (in an issue-rate probe on gfx950 dot4 and
-// the other VOP3 forms took twice as long as a plain add; on the M=4 headline
-// shape the change was worth 78 % -> 82 % of HBM peak in batched launches).
-// A field holds at most 257 entries (257 * 255 < 65536);
-// flush() widens the fields into acc[] and has to be called at least that often.
+// the other VOP3 forms took twice as long as a plain add).
+// A 16-bit sum holds at most 257 entries (257 * 255 < 65536);
+// flush() widens the sums into acc[] and has to be called at least that often.
 // Both signs of a lane always gather the same number of entries, so the bias cancels.
 template <typename Act, int MT> struct Sums {
     typedef typename Acc<Act>::type A;
     static constexpr bool SWAR = sizeof(Act) == 1 && MT > 1;
     static constexpr int NW = SWAR ? MT / 4 : 1;
     A acc[MT];
-    u32 lo[2][NW], hi[2][NW];  // [sign][dword]: rows 4j / 4j+2 and rows 4j+1 / 4j+3 (SWAR only)
+    u32 lo[2][NW], hi[2][NW];  // [sign][dword]: rows 4j / 4j+2 in 16-bit fields, and the sum of the dwords >> 8 (SWAR only)
 
     __device__ __forceinline__ void init()
     {
@@ -77,7 +78,7 @@ template <typename Act, int MT> struct Sums {
 #pragma unroll
             for (int j = 0; j < NW; ++j) {
                 lo[NEG][j] += r.v[j] & 0x00ff00ffu;
-                hi[NEG][j] += (r.v[j] >> 8) & 0x00ff00ffu;
+                hi[NEG][j] += r.v[j] >> 8;
             }
         } else {
 #pragma unroll
@@ -104,10 +105,12 @@ template <typename Act, int MT> struct Sums {
         if constexpr (SWAR) {
 #pragma unroll
             for (int j = 0; j < NW; ++j) {
+                // hi = sum(b1) + 2^8 sum(b2) + 2^16 sum(b3) mod 2^32; take sum(b2) out and two 16-bit sums remain
+                const u32 p13 = hi[0][j] - ((lo[0][j] >> 16) << 8), n13 = hi[1][j] - ((lo[1][j] >> 16) << 8);
                 acc[4 * j + 0] += (int)(lo[0][j] & 0xffffu) - (int)(lo[1][j] & 0xffffu);
-                acc[4 * j + 1] += (int)(hi[0][j] & 0xffffu) - (int)(hi[1][j] & 0xffffu);
+                acc[4 * j + 1] += (int)(p13 & 0xffffu) - (int)(n13 & 0xffffu);
                 acc[4 * j + 2] += (int)(lo[0][j] >> 16) - (int)(lo[1][j] >> 16);
-                acc[4 * j + 3] += (int)(hi[0][j] >> 16) - (int)(hi[1][j] >> 16);
+                acc[4 * j + 3] += (int)(p13 >> 16) - (int)(n13 >> 16);
                 lo[0][j] = hi[0][j] = lo[1][j] = hi[1][j] = 0u;
             }
         }
