@@ -34,6 +34,10 @@ template <typename Act, int MT> __host__ __device__ constexpr int slot_bytes()
 __host__ __device__ constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v >> 1); }
 
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
+typedef int v4i __attribute__((ext_vector_type(4)));
+#ifndef SPTMM_MX
+#define SPTMM_MX 1
+#endif
 
 // The running sums of one lane: acc[m] (+|-)= X[m][k] for every gathered row k.
 // int8 activations with MT > 1 keep the tile's bytes biased by 128 (unsigned) and
@@ -50,6 +54,10 @@ template <typename Act, int MT> struct Sums {
     typedef typename Acc<Act>::type A;
     static constexpr bool SWAR = sizeof(Act) == 1 && MT > 1;
     static constexpr int NW = SWAR ? MT / 4 : 1;
+    static constexpr bool MX = SWAR && SPTMM_MX;            // sums on the matrix unit
+    static constexpr int ND = MX ? MT / 4 : 1;
+    static constexpr u32 BIAS = SWAR && !MX ? 0x80808080u : 0u;  // what the tile's bytes are stored xor'ed with
+    v4i D[ND], Bp[ND], Bn[ND];                               // MX: 16x16 int32 result tiles and the +1 / -1 selectors
     A acc[MT];
     u32 lo[2][NW], hi[2][NW];  // [sign][dword]: rows 4j / 4j+2 in 16-bit fields, and the sum of the dwords >> 8 (SWAR only)
 
@@ -57,7 +65,28 @@ template <typename Act, int MT> struct Sums {
     {
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[m] = (A)0;
-        if constexpr (SWAR) {
+        if constexpr (MX) {
+            // Selector held by lane j + 16 g (k-block g, output column j): 1 where the byte of the A operand
+            // at the same (g, byte) position is to be added into column j.  MT = 4: A = 4 entries x 4 rows,
+            // column 4 g + row.  MT = 8: A = 2 entries x 8 rows, tile x takes k-blocks 2x and 2x + 1, column
+            // 8 (g & 1) + row.
+            const int l = threadIdx.x & 63, g = l >> 4, j = l & 15;
+            const u32 b = 1u << (8 * (j & 3));
+#pragma unroll
+            for (int x = 0; x < ND; ++x) {
+                u32 e, o;
+                if constexpr (MT == 4) {
+                    e = o = (j >> 2) == g ? b : 0u;
+                } else {
+                    const bool on = (g >> 1) == x && (j >> 3) == (g & 1);
+                    e = on && !(j & 4) ? b : 0u;
+                    o = on && (j & 4) ? b : 0u;
+                }
+                Bp[x] = v4i{(int)e, (int)o, (int)e, (int)o};
+                Bn[x] = v4i{(int)(e * 255u), (int)(o * 255u), (int)(e * 255u), (int)(o * 255u)};
+                D[x] = v4i{0, 0, 0, 0};
+            }
+        } else if constexpr (SWAR) {
 #pragma unroll
             for (int j = 0; j < NW; ++j) lo[0][j] = hi[0][j] = lo[1][j] = hi[1][j] = 0u;
         }
@@ -86,12 +115,38 @@ template <typename Act, int MT> struct Sums {
         }
     }
 
+    // NE gathered slots of one sign.  MX: four entries (MT = 8: two) form the 16 bytes a lane gives to one
+    // v_mfma_i32_16x16x64_i8; the product with the selector adds every byte into the int32 of its
+    // (lane, row) -- the adds of the masked-field code, on the matrix unit, which this kernel leaves idle.
+    template <bool NEG, int NE> __device__ __forceinline__ void accum_n(const Raw *r)
+    {
+        if constexpr (MX) {
+            constexpr int PER = 16 / MT;  // entries per operand
+#pragma unroll
+            for (int e = 0; e < NE; e += PER) {
+                v4i a;
+                if constexpr (MT == 4)
+                    a = v4i{(int)r[e].v[0], e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[0] : 0, e + 2 < NE ? (int)r[e + 2 < NE ? e + 2 : e].v[0] : 0,
+                            e + 3 < NE ? (int)r[e + 3 < NE ? e + 3 : e].v[0] : 0};
+                else
+                    a = v4i{(int)r[e].v[0], (int)r[e].v[1], e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[0] : 0,
+                            e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[1] : 0};
+#pragma unroll
+                for (int x = 0; x < ND; ++x) D[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[x] : Bp[x], D[x], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < NE; ++e) accum<NEG>(r[e]);
+        }
+    }
+
     // Pin the sums once per round.  Integer adds may be reassociated freely, and without
     // this the compiler keeps every gathered value of every round alive to sum them in
     // one tree at the end.
     __device__ __forceinline__ void pin()
     {
-        if constexpr (SWAR) {
+        if constexpr (MX) {
+        } else if constexpr (SWAR) {
 #pragma unroll
             for (int j = 0; j < NW; ++j) asm volatile("" : "+v"(lo[0][j]), "+v"(hi[0][j]), "+v"(lo[1][j]), "+v"(hi[1][j]));
         } else {
@@ -102,7 +157,7 @@ template <typename Act, int MT> struct Sums {
 
     __device__ __forceinline__ void flush()
     {
-        if constexpr (SWAR) {
+        if constexpr (SWAR && !MX) {
 #pragma unroll
             for (int j = 0; j < NW; ++j) {
                 // hi = sum(b1) + 2^8 sum(b2) + 2^16 sum(b3) mod 2^32; take sum(b2) out and two 16-bit sums remain
@@ -189,8 +244,7 @@ __device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &ru
     constexpr int NE = NBYTES / Flavour<MODE>::ESZ;
     typename Sums<Act, MT>::Raw r[NE];
     fetch<Act, MT, MODE, PRE, NBYTES>(lds, d, run, r);
-#pragma unroll
-    for (int e = 0; e < NE; ++e) acc.template accum<NEG>(r[e]);
+    acc.template accum_n<NEG, NE>(r);
 }
 
 template <typename Act, int MT, int MODE, bool PRE, bool NEG>
@@ -202,8 +256,7 @@ __device__ __forceinline__ void consume16(const unsigned char *lds, const uint4 
     fetch<Act, MT, MODE, PRE, 4>(lds, v.y, run, r + NE);
     fetch<Act, MT, MODE, PRE, 4>(lds, v.z, run, r + 2 * NE);
     fetch<Act, MT, MODE, PRE, 4>(lds, v.w, run, r + 3 * NE);
-#pragma unroll
-    for (int e = 0; e < 4 * NE; ++e) acc.template accum<NEG>(r[e]);
+    acc.template accum_n<NEG, 4 * NE>(r);
 }
 
 // 4 rows x 4 consecutive k (one dword per row) -> 4 dwords, dword j = the 4 rows at k+j
@@ -255,7 +308,7 @@ template <typename Act, int MT> struct Stager {
             for (int j = 0; j < 4; ++j) {
                 u32 o[4], q[4];
                 transpose4x4(comp(r[0], j), comp(r[1], j), comp(r[2], j), comp(r[3], j), o);
-                constexpr u32 B = 0x80808080u;  // bytes are stored biased by 128 (see Sums)
+                constexpr u32 B = Sums<Act, MT>::BIAS;  // the masked-field sums take the bytes biased by 128 (see Sums)
                 if constexpr (MT == 4) {
                     t[4 * item + j] = make_uint4(o[0] ^ B, o[1] ^ B, o[2] ^ B, o[3] ^ B);
                 } else {
@@ -295,6 +348,8 @@ template <typename Act, int MT> struct Stager {
 template <int CTRL> __device__ __forceinline__ int dpp(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
 template <int CTRL> __device__ __forceinline__ float dpp(float v) { return __builtin_bit_cast(float, dpp<CTRL>(__builtin_bit_cast(int, v))); }
 __device__ __forceinline__ int swz16(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401f); }  // lane ^ 16
+__device__ __forceinline__ int swz8(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x201f); }   // lane ^ 8
+__device__ __forceinline__ int swz4(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x101f); }   // lane ^ 4
 __device__ __forceinline__ float swz16(float v) { return __builtin_bit_cast(float, swz16(__builtin_bit_cast(int, v))); }
 
 // Sum over groups of 2^logL consecutive lanes (logL >= 2); every lane of a group ends with the group's total.
@@ -565,9 +620,9 @@ struct ListsBody {
                 St::store(smem, item, r);
             }
         }
-        // rows K.. read as zero (biased bytes: 128)
+        // rows K.. read as zero
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
-            reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = Sums<Act, MT>::SWAR ? 0x80808080u : 0u;
+            reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = Sums<Act, MT>::BIAS;
         __syncthreads();
 
         A *C = reinterpret_cast<A *>(p.C);
@@ -704,27 +759,77 @@ struct ListsBody {
             }
 
             acc.flush();  // since the last one: at most 10 rounds and the tail, 175 entries per sign
+            if constexpr (Sums<Act, MT>::MX) {
+                // Result tile x, lane l, register r: the sum of source lane 16 g + 4 (l >> 4) + r and row m, where
+                // MT = 4: g = (l >> 2) & 3, m = l & 3;  MT = 8: g = 2 x + ((l >> 3) & 1), m = l & 7.
+                // The four registers are neighbouring lanes of one column; the rest of a column's L lanes is
+                // spread over lane bits 4, 5 (the quarter) and, from L = 32, the bits that hold g.
+                constexpr int ND = MT / 4;
+                const int logL = p.logL;
+                int t[ND];
 #pragma unroll
-            for (int m = 0; m < MT; ++m) acc.acc[m] = lanes_sum(acc.acc[m], p.logL);
-
-            if (p.W == 1) {
-                if (active && (lane & (L - 1)) == 0) {
-                    const int col = (task << (6 - p.logL)) + (lane >> p.logL);
+                for (int x = 0; x < ND; ++x) {
+                    t[x] = acc.D[x][0] + acc.D[x][1] + acc.D[x][2] + acc.D[x][3];
+                    t[x] += swz16(t[x]);
+                    if (logL >= 4) t[x] += __shfl_xor(t[x], 32, 64);
+                    if (logL >= 5) t[x] += MT == 4 ? swz4(t[x]) : swz8(t[x]);
+                }
+                if constexpr (MT == 4) {
+                    if (logL >= 6) t[0] += swz8(t[0]);
+                } else {
+                    if (logL >= 6) t[0] += t[1];
+                }
+                const int m = lane & (MT - 1);
+                int col[ND];
+                bool writer;
+                if constexpr (MT == 4) {
+                    const int g = (lane >> 2) & 3;
+                    writer = logL == 3 ? !(lane & 16) : logL == 4 ? lane < 16 : logL == 5 ? (lane < 16 && !(lane & 4)) : lane < 4;
+                    col[0] = logL == 3 ? 2 * g + (lane >> 5) : logL == 4 ? g : logL == 5 ? g >> 1 : 0;
+                } else {
+                    const int g = (lane >> 3) & 1;
+                    writer = logL == 3 ? !(lane & 16) : logL == 4 ? lane < 16 : lane < 8;
+                    col[0] = logL == 3 ? 2 * g + (lane >> 5) : logL == 4 ? g : 0;
+                    col[1] = logL == 3 ? 4 + 2 * g + (lane >> 5) : logL == 4 ? 2 + g : 1;
+                }
+                if (p.W == 1) {
+                    if (active && writer && m0 + m < p.M) {
+                        const int cbase = task << (6 - logL);
+                        const float bk = QUANT ? qinv[m] : 0.f;
 #pragma unroll
-                    for (int m = 0; m < MT; ++m)
-                        if (m0 + m < p.M) {
+                        for (int x = 0; x < ND; ++x) {
+                            if (x > 0 && logL >= 6) break;  // one column per task: tile 1 is already in t[0]
                             if constexpr (QUANT)
-                                Cf[(size_t)(m0 + m) * p.N + col] = (float)acc.acc[m] * back[m] * p.w_scale;
+                                Cf[(size_t)(m0 + m) * p.N + cbase + col[x]] = (float)t[x] * bk * p.w_scale;
                             else
-                                C[(size_t)(m0 + m) * p.N + col] = acc.acc[m];
+                                C[(size_t)(m0 + m) * p.N + cbase + col[x]] = t[x];
                         }
+                    }
+                } else if (lane < MT) {
+                    part[wave * MT + lane] = t[0];
                 }
             } else {
-                // second pass: the W wavefronts of a column meet in a small LDS buffer
-                if (lane == 0) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m) acc.acc[m] = lanes_sum(acc.acc[m], p.logL);
+                if (p.W == 1) {
+                    if (active && (lane & (L - 1)) == 0) {
+                        const int col = (task << (6 - p.logL)) + (lane >> p.logL);
+#pragma unroll
+                        for (int m = 0; m < MT; ++m)
+                            if (m0 + m < p.M) {
+                                if constexpr (QUANT)
+                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)acc.acc[m] * back[m] * p.w_scale;
+                                else
+                                    C[(size_t)(m0 + m) * p.N + col] = acc.acc[m];
+                            }
+                    }
+                } else if (lane == 0) {
 #pragma unroll
                     for (int m = 0; m < MT; ++m) part[wave * MT + m] = acc.acc[m];
                 }
+            }
+            if (p.W != 1) {
+                // second pass: the W wavefronts of a column meet in a small LDS buffer
                 __syncthreads();
                 if (active && lane == 0 && (wave & (p.W - 1)) == 0) {
                     const int col = task / p.W;
