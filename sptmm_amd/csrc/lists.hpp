@@ -35,31 +35,25 @@ __host__ __device__ constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v
 
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 typedef int v4i __attribute__((ext_vector_type(4)));
-#ifndef SPTMM_MX
-#define SPTMM_MX 1
-#endif
 
 // The running sums of one lane: acc[m] (+|-)= X[m][k] for every gathered row k.
-// int8 activations with MT > 1 keep the tile's bytes biased by 128 (unsigned) and
-// add them four rows at a time into plain 32-bit registers: bytes 0 and 2 masked
-// into two 16-bit fields, and the whole dword shifted right by 8, whose running sum
-// sum(b1) + 2^8 sum(b2) + 2^16 sum(b3) (mod 2^32) separates again once sum(b2) is
-// known -- a mask, a shift and two adds per four rows in place of four dot4
-// instructions with one-hot selectors (in an issue-rate probe on gfx950 dot4 and
-// the other VOP3 forms took twice as long as a plain add).
-// A 16-bit sum holds at most 257 entries (257 * 255 < 65536);
-// flush() widens the sums into acc[] and has to be called at least that often.
-// Both signs of a lane always gather the same number of entries, so the bias cancels.
+//
+// int8 activations with MT > 1 (MX): a gathered slot holds the MT rows of one index as packed
+// bytes, and adding bytes into per-row int32 sums on the VALU costs one instruction per entry
+// and row however it is arranged (masked 16-bit fields: 4 per four rows; SDWA byte adds and
+// 16-bit-field tiles measured slower) -- from M = 4 that, not HBM, set the time.  The matrix unit
+// does the same adds: four entries (MT = 8: two) are the 16 bytes a lane hands to one
+// v_mfma_i32_16x16x64_i8 as the A operand, and the B operand is a constant selector of 0 / 1
+// (-1 for the minus list) that routes every byte to the int32 of its (lane, row) in the 16x16
+// result.  Nothing is contracted -- each output sums one lane's own bytes of one row -- the
+// instruction is used as 256 byte-to-int32 adders, on a unit this kernel otherwise leaves idle.
 template <typename Act, int MT> struct Sums {
     typedef typename Acc<Act>::type A;
-    static constexpr bool SWAR = sizeof(Act) == 1 && MT > 1;
-    static constexpr int NW = SWAR ? MT / 4 : 1;
-    static constexpr bool MX = SWAR && SPTMM_MX;            // sums on the matrix unit
-    static constexpr int ND = MX ? MT / 4 : 1;
-    static constexpr u32 BIAS = SWAR && !MX ? 0x80808080u : 0u;  // what the tile's bytes are stored xor'ed with
-    v4i D[ND], Bp[ND], Bn[ND];                               // MX: 16x16 int32 result tiles and the +1 / -1 selectors
+    static constexpr bool MX = sizeof(Act) == 1 && MT > 1;  // sums on the matrix unit
+    static constexpr int NW = MX ? MT / 4 : 1;              // dwords per gathered slot (int8)
+    static constexpr int ND = MX ? MT / 4 : 1;              // result tiles
+    v4i D[ND], Bp[ND], Bn[ND];                              // MX: 16x16 int32 result tiles and the +1 / -1 selectors
     A acc[MT];
-    u32 lo[2][NW], hi[2][NW];  // [sign][dword]: rows 4j / 4j+2 in 16-bit fields, and the sum of the dwords >> 8 (SWAR only)
 
     __device__ __forceinline__ void init()
     {
@@ -86,9 +80,6 @@ template <typename Act, int MT> struct Sums {
                 Bn[x] = v4i{(int)(e * 255u), (int)(o * 255u), (int)(e * 255u), (int)(o * 255u)};
                 D[x] = v4i{0, 0, 0, 0};
             }
-        } else if constexpr (SWAR) {
-#pragma unroll
-            for (int j = 0; j < NW; ++j) lo[0][j] = hi[0][j] = lo[1][j] = hi[1][j] = 0u;
         }
     }
 
@@ -99,29 +90,11 @@ template <typename Act, int MT> struct Sums {
     // the slot at byte offset `addr` of the tile
     static __device__ __forceinline__ Raw load(const unsigned char *lds, u32 addr) { return *reinterpret_cast<const Raw *>(lds + addr); }
 
-    template <bool NEG> __device__ __forceinline__ void accum(const Raw &r)
-    {
-        if constexpr (sizeof(Act) == 1 && MT == 1) {
-            acc[0] = NEG ? acc[0] - (int)r.v[0] : acc[0] + (int)r.v[0];
-        } else if constexpr (SWAR) {
-#pragma unroll
-            for (int j = 0; j < NW; ++j) {
-                lo[NEG][j] += r.v[j] & 0x00ff00ffu;
-                hi[NEG][j] += r.v[j] >> 8;
-            }
-        } else {
-#pragma unroll
-            for (int m = 0; m < MT; ++m) acc[m] = NEG ? acc[m] - (float)r.v[m] : acc[m] + (float)r.v[m];
-        }
-    }
-
-    // NE gathered slots of one sign.  MX: four entries (MT = 8: two) form the 16 bytes a lane gives to one
-    // v_mfma_i32_16x16x64_i8; the product with the selector adds every byte into the int32 of its
-    // (lane, row) -- the adds of the masked-field code, on the matrix unit, which this kernel leaves idle.
+    // NE gathered slots of one sign
     template <bool NEG, int NE> __device__ __forceinline__ void accum_n(const Raw *r)
     {
         if constexpr (MX) {
-            constexpr int PER = 16 / MT;  // entries per operand
+            constexpr int PER = 16 / MT;  // entries per A operand; a short tail is filled with zero bytes
 #pragma unroll
             for (int e = 0; e < NE; e += PER) {
                 v4i a;
@@ -136,38 +109,25 @@ template <typename Act, int MT> struct Sums {
             }
         } else {
 #pragma unroll
-            for (int e = 0; e < NE; ++e) accum<NEG>(r[e]);
+            for (int e = 0; e < NE; ++e) {
+                if constexpr (sizeof(Act) == 1) {
+                    acc[0] = NEG ? acc[0] - (int)r[e].v[0] : acc[0] + (int)r[e].v[0];
+                } else {
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) acc[m] = NEG ? acc[m] - (float)r[e].v[m] : acc[m] + (float)r[e].v[m];
+                }
+            }
         }
     }
 
     // Pin the sums once per round.  Integer adds may be reassociated freely, and without
     // this the compiler keeps every gathered value of every round alive to sum them in
-    // one tree at the end.
+    // one tree at the end.  (The matrix-unit sums are chained by their accumulator.)
     __device__ __forceinline__ void pin()
     {
-        if constexpr (MX) {
-        } else if constexpr (SWAR) {
-#pragma unroll
-            for (int j = 0; j < NW; ++j) asm volatile("" : "+v"(lo[0][j]), "+v"(hi[0][j]), "+v"(lo[1][j]), "+v"(hi[1][j]));
-        } else {
+        if constexpr (!MX) {
 #pragma unroll
             for (int m = 0; m < MT; ++m) asm volatile("" : "+v"(acc[m]));
-        }
-    }
-
-    __device__ __forceinline__ void flush()
-    {
-        if constexpr (SWAR && !MX) {
-#pragma unroll
-            for (int j = 0; j < NW; ++j) {
-                // hi = sum(b1) + 2^8 sum(b2) + 2^16 sum(b3) mod 2^32; take sum(b2) out and two 16-bit sums remain
-                const u32 p13 = hi[0][j] - ((lo[0][j] >> 16) << 8), n13 = hi[1][j] - ((lo[1][j] >> 16) << 8);
-                acc[4 * j + 0] += (int)(lo[0][j] & 0xffffu) - (int)(lo[1][j] & 0xffffu);
-                acc[4 * j + 1] += (int)(p13 & 0xffffu) - (int)(n13 & 0xffffu);
-                acc[4 * j + 2] += (int)(lo[0][j] >> 16) - (int)(lo[1][j] >> 16);
-                acc[4 * j + 3] += (int)(p13 >> 16) - (int)(n13 >> 16);
-                lo[0][j] = hi[0][j] = lo[1][j] = hi[1][j] = 0u;
-            }
         }
     }
 };
@@ -270,6 +230,25 @@ __device__ __forceinline__ void transpose4x4(u32 r0, u32 r1, u32 r2, u32 r3, u32
     o[3] = __builtin_amdgcn_perm(d, b, 0x07060302u);
 }
 
+// The same with the two output pairs exchanged where `odd`: o[0], o[1] = k+2, k+3 and o[2], o[3] = k, k+1.
+// The byte selectors come from registers, so the exchange costs no instruction.
+__device__ __forceinline__ void transpose4x4_swap(u32 r0, u32 r1, u32 r2, u32 r3, bool odd, u32 (&o)[4])
+{
+    const u32 s0 = odd ? 0x07030602u : 0x05010400u, s1 = odd ? 0x05010400u : 0x07030602u;
+    u32 a = __builtin_amdgcn_perm(r1, r0, s0), b = __builtin_amdgcn_perm(r1, r0, s1);
+    u32 c = __builtin_amdgcn_perm(r3, r2, s0), d = __builtin_amdgcn_perm(r3, r2, s1);
+    o[0] = __builtin_amdgcn_perm(c, a, 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(c, a, 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(d, b, 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(d, b, 0x07060302u);
+}
+__device__ __forceinline__ void swap_if(bool c, u32 &a, u32 &b)
+{
+    const u32 x = c ? b : a, y = c ? a : b;
+    a = x;
+    b = y;
+}
+
 __device__ __forceinline__ u32 comp(const uint4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
 __device__ __forceinline__ u32 f2u(float f) { return __builtin_bit_cast(u32, f); }
 __device__ __forceinline__ float h2f(u32 d, int hi) { return (float)__builtin_bit_cast(_Float16, (unsigned short)(hi ? d >> 16 : d & 0xffffu)); }
@@ -303,19 +282,38 @@ template <typename Act, int MT> struct Stager {
                 int d = (int)comp(r[0], j);
                 t[4 * item + j] = make_uint4((u32)((d << 24) >> 24), (u32)((d << 16) >> 24), (u32)((d << 8) >> 24), (u32)(d >> 24));
             }
-        } else if constexpr (sizeof(Act) == 1) {  // [k][MT bytes]
+        } else if constexpr (sizeof(Act) == 1 && MT == 4) {  // [k][4 bytes]
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                u32 o[4], q[4];
+                u32 o[4];
                 transpose4x4(comp(r[0], j), comp(r[1], j), comp(r[2], j), comp(r[3], j), o);
-                constexpr u32 B = Sums<Act, MT>::BIAS;  // the masked-field sums take the bytes biased by 128 (see Sums)
-                if constexpr (MT == 4) {
-                    t[4 * item + j] = make_uint4(o[0] ^ B, o[1] ^ B, o[2] ^ B, o[3] ^ B);
-                } else {
-                    transpose4x4(comp(r[4], j), comp(r[5], j), comp(r[6], j), comp(r[7], j), q);
-                    t[2 * (4 * item + j)] = make_uint4(o[0] ^ B, q[0] ^ B, o[1] ^ B, q[1] ^ B);
-                    t[2 * (4 * item + j) + 1] = make_uint4(o[2] ^ B, q[2] ^ B, o[3] ^ B, q[3] ^ B);
-                }
+                t[4 * item + j] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        } else if constexpr (sizeof(Act) == 1) {  // [k][8 bytes]
+            // An item is 128 bytes of the tile, so the lanes of a 16-byte write all start on the same bank
+            // and the write takes eight passes (counted: three quarters of this kernel's LDS conflict
+            // cycles at K = 13824).  Lane `item` therefore writes its eight 16-byte chunks in the order
+            // c ^ (item & 7): eight neighbouring lanes then cover eight different chunks.  Bit 0 of the
+            // order is an exchange of byte selectors in the transposition, bits 1-2 a conditional
+            // exchange of the loaded dwords.
+            const u32 rho = (u32)item & 7u;
+            u32 x[8][4];
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) x[m][j] = comp(r[m], j);
+                swap_if(rho & 2u, x[m][0], x[m][1]);
+                swap_if(rho & 2u, x[m][2], x[m][3]);
+                swap_if(rho & 4u, x[m][0], x[m][2]);
+                swap_if(rho & 4u, x[m][1], x[m][3]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {  // x[m][j] = dword j ^ (rho >> 1) of row m
+                u32 o[4], q[4];
+                transpose4x4_swap(x[0][j], x[1][j], x[2][j], x[3][j], rho & 1u, o);
+                transpose4x4_swap(x[4][j], x[5][j], x[6][j], x[7][j], rho & 1u, q);
+                t[8 * item + ((2 * j) ^ rho)] = make_uint4(o[0], q[0], o[1], q[1]);
+                t[8 * item + ((2 * j + 1) ^ rho)] = make_uint4(o[2], q[2], o[3], q[3]);
             }
         } else if constexpr (sizeof(Act) == 2 && MT == 1) {  // 16 halves -> 16 floats
 #pragma unroll
@@ -622,7 +620,7 @@ struct ListsBody {
         }
         // rows K.. read as zero
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
-            reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = Sums<Act, MT>::BIAS;
+            reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = 0u;
         __syncthreads();
 
         A *C = reinterpret_cast<A *>(p.C);
@@ -710,7 +708,6 @@ struct ListsBody {
                         eat(smem, buf[i], runp, runq, acc);
                         buf[i] = load_round(wp, base + RING + i);
                     }
-                    acc.flush();  // at most 8 rounds = 128 entries per sign since the last one
                 }
                 if (R - base > RING) {
 #pragma unroll
@@ -720,7 +717,6 @@ struct ListsBody {
                         buf[i] = load_round(wp, r < R ? r : R - 1);
                     }
                     base += RING;
-                    acc.flush();
                 }
 #pragma unroll
                 for (int i = 0; i < RING; ++i) {
@@ -758,7 +754,6 @@ struct ListsBody {
                 }
             }
 
-            acc.flush();  // since the last one: at most 10 rounds and the tail, 175 entries per sign
             if constexpr (Sums<Act, MT>::MX) {
                 // Result tile x, lane l, register r: the sum of source lane 16 g + 4 (l >> 4) + r and row m, where
                 // MT = 4: g = (l >> 2) & 3, m = l & 3;  MT = 8: g = 2 x + ((l >> 3) & 1), m = l & 7.
