@@ -35,6 +35,8 @@ __host__ __device__ constexpr int ilog2(int v) { return v <= 1 ? 0 : 1 + ilog2(v
 
 template <typename T, int N> struct alignas(sizeof(T) * N) Vec { T v[N]; };
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 // The running sums of one lane: acc[m] (+|-)= X[m][k] for every gathered row k.
 //
@@ -50,10 +52,23 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 template <typename Act, int MT> struct Sums {
     typedef typename Acc<Act>::type A;
     static constexpr bool MX = sizeof(Act) == 1 && MT > 1;  // sums on the matrix unit
+    static constexpr bool MXF = sizeof(Act) == 2 && MT > 1; // the same for fp16 rows (MT = 4): v_mfma_f32_16x16x32_f16,
+                                                            // two entries x four rows per operand, selector of 0 / +-1.0
     static constexpr int NW = MX ? MT / 4 : 1;              // dwords per gathered slot (int8)
     static constexpr int ND = MX ? MT / 4 : 1;              // result tiles
     v4i D[ND], Bp[ND], Bn[ND];                              // MX: 16x16 int32 result tiles and the +1 / -1 selectors
+    v4f Df;                                                 // MXF: the fp32 result tile ...
+    v8h Bpf, Bnf;                                           // ... and its selectors
     A acc[MT];
+
+    // sum of the four registers a lane holds of result tile x
+    __device__ __forceinline__ A tile_sum(int x) const
+    {
+        if constexpr (MXF)
+            return (Df[0] + Df[1]) + (Df[2] + Df[3]);
+        else
+            return (A)(D[x][0] + D[x][1] + D[x][2] + D[x][3]);
+    }
 
     __device__ __forceinline__ void init()
     {
@@ -80,6 +95,15 @@ template <typename Act, int MT> struct Sums {
                 Bn[x] = v4i{(int)(e * 255u), (int)(o * 255u), (int)(e * 255u), (int)(o * 255u)};
                 D[x] = v4i{0, 0, 0, 0};
             }
+        } else if constexpr (MXF) {
+            const int l = threadIdx.x & 63, g = l >> 4, j = l & 15;
+#pragma unroll
+            for (int y = 0; y < 8; ++y) {
+                const bool on = (j >> 2) == g && (y & 3) == (j & 3);
+                Bpf[y] = on ? (_Float16)1.0f : (_Float16)0.0f;
+                Bnf[y] = on ? (_Float16)-1.0f : (_Float16)0.0f;
+            }
+            Df = v4f{0.f, 0.f, 0.f, 0.f};
         }
     }
 
@@ -107,6 +131,17 @@ template <typename Act, int MT> struct Sums {
 #pragma unroll
                 for (int x = 0; x < ND; ++x) D[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[x] : Bp[x], D[x], 0, 0, 0);
             }
+        } else if constexpr (MXF) {
+#pragma unroll
+            for (int e = 0; e < NE; e += 2) {
+                v8h a;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    a[m] = r[e].v[m];
+                    a[4 + m] = e + 1 < NE ? r[e + 1 < NE ? e + 1 : e].v[m] : (_Float16)0.0f;
+                }
+                Df = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf : Bpf, Df, 0, 0, 0);
+            }
         } else {
 #pragma unroll
             for (int e = 0; e < NE; ++e) {
@@ -125,7 +160,7 @@ template <typename Act, int MT> struct Sums {
     // one tree at the end.  (The matrix-unit sums are chained by their accumulator.)
     __device__ __forceinline__ void pin()
     {
-        if constexpr (!MX) {
+        if constexpr (!MX && !MXF) {
 #pragma unroll
             for (int m = 0; m < MT; ++m) asm volatile("" : "+v"(acc[m]));
         }
@@ -349,6 +384,8 @@ __device__ __forceinline__ int swz16(int v) { return __builtin_amdgcn_ds_swizzle
 __device__ __forceinline__ int swz8(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x201f); }   // lane ^ 8
 __device__ __forceinline__ int swz4(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x101f); }   // lane ^ 4
 __device__ __forceinline__ float swz16(float v) { return __builtin_bit_cast(float, swz16(__builtin_bit_cast(int, v))); }
+__device__ __forceinline__ float swz8(float v) { return __builtin_bit_cast(float, swz8(__builtin_bit_cast(int, v))); }
+__device__ __forceinline__ float swz4(float v) { return __builtin_bit_cast(float, swz4(__builtin_bit_cast(int, v))); }
 
 // Sum over groups of 2^logL consecutive lanes (logL >= 2); every lane of a group ends with the group's total.
 template <typename T>
@@ -754,17 +791,17 @@ struct ListsBody {
                 }
             }
 
-            if constexpr (Sums<Act, MT>::MX) {
+            if constexpr (Sums<Act, MT>::MX || Sums<Act, MT>::MXF) {
                 // Result tile x, lane l, register r: the sum of source lane 16 g + 4 (l >> 4) + r and row m, where
                 // MT = 4: g = (l >> 2) & 3, m = l & 3;  MT = 8: g = 2 x + ((l >> 3) & 1), m = l & 7.
                 // The four registers are neighbouring lanes of one column; the rest of a column's L lanes is
                 // spread over lane bits 4, 5 (the quarter) and, from L = 32, the bits that hold g.
-                constexpr int ND = MT / 4;
+                constexpr int ND = Sums<Act, MT>::ND;
                 const int logL = p.logL;
-                int t[ND];
+                A t[ND];
 #pragma unroll
                 for (int x = 0; x < ND; ++x) {
-                    t[x] = acc.D[x][0] + acc.D[x][1] + acc.D[x][2] + acc.D[x][3];
+                    t[x] = acc.tile_sum(x);
                     t[x] += swz16(t[x]);
                     if (logL >= 4) t[x] += __shfl_xor(t[x], 32, 64);
                     if (logL >= 5) t[x] += MT == 4 ? swz4(t[x]) : swz8(t[x]);
