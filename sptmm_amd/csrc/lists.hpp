@@ -443,7 +443,7 @@ __device__ __forceinline__ Round load_round(const uint4 *wp, int r)
 // q = clamp(rint(x * s), -127, 127)) for the kernels that take fp16 / bf16 rows and
 // hand back floats.  Item = 16 consecutive k of all MT rows, as in Stager.
 template <int MT> struct Quantiser {
-    static constexpr int HOLD = MT == 1 ? 2 : 0;  // items a thread keeps in registers between the two passes (the rest is read twice)
+    static constexpr int HOLD = MT <= 4 ? 2 : 0;  // items a thread keeps in registers between the two passes (the rest is read twice)
     typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
     // 2 x 16 bytes per row: the item's 16 values of row m0 + m (rows past M read as zero)
