@@ -71,9 +71,10 @@ def main():
     ap.add_argument("--steps", type=int, default=256, help="timed steps; one step = one launch of BATCH GEMVs")
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--legs", default="single,others,ceiling",
+    ap.add_argument("--legs", default="single,others,ceiling,m4",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, "
-                         "sync-each-call), others (delta and i2s encodings), copy (4 launches of a 1 GiB copy kernel, for counter "
+                         "sync-each-call), others (delta and i2s encodings), m4 (config 1: the same matrix at M=4, all three "
+                         "encodings), copy (4 launches of a 1 GiB copy kernel, for counter "
                          "calibration), ceiling (a pure streaming read of as many bytes as one step moves: the practical HBM read "
                          "ceiling on this box); profiling runs use --legs none or --legs copy")
     a = ap.parse_args()
@@ -183,6 +184,40 @@ def main():
             for c in cps:
                 c.free()
 
+    m4 = {}
+    if "m4" in legs:
+        # config 1: the same matrix at four activation rows (indices still read once per GEMV)
+        M4 = 4
+        X4 = sp.make_x_i8(0xC0FFEE ^ M4, M4, K)
+        x4 = sp.DeviceBuffer.from_numpy(X4)
+        c4 = sp.DeviceBuffer(4 * M4 * N * BATCH)
+        ref4 = None
+        for name, mk, ncp in (("u16_split32", lambda: sp.Weights.upload_u16(pos, neg, K, SPLIT), BATCH),
+                              ("delta8_split16", lambda: sp.Weights.upload_delta(pos, neg, K, 16), 2 * BATCH),
+                              ("i2s", lambda: sp.Weights.upload_i2s(Wd), 4 * BATCH)):
+            ww = mk()
+            got = ww.matmul(X4)
+            ref4 = got if ref4 is None else ref4
+            assert (got == ref4).all(), name
+            cps = [ww] + [ww.clone() for _ in range(ncp - 1)]
+            b = algorithmic_bytes(ww.nbytes, M4)
+            sp.measure_gemv(cps, 0, x4, M4, c4, 256, 0, st)
+            r = {"bytes": b, "single_cold_us": round(sp.measure_gemv(cps, 0, x4, M4, c4, 4096, 0, st), 3)}
+            sp.measure_gemv(cps[:1], 0, x4, M4, c4, 256, 0, st)
+            r["single_warm_us"] = round(sp.measure_gemv(cps[:1], 0, x4, M4, c4, 4096, 0, st), 3)
+            groups = [cps[i:i + BATCH] for i in range(0, len(cps), BATCH)]
+            for g in groups:
+                sp.measure_gemv(g, 0, x4, M4, c4, BATCH * max(a.warmup // len(groups), 1), 3, st)
+            t = [sp.measure_gemv(g, 0, x4, M4, c4, BATCH * max(a.steps // len(groups), 1), 3, st) for g in groups]
+            r["batched_cold_us"] = round(sum(t) / len(t), 3)
+            r["batched_cold_gbps"] = round(b / r["batched_cold_us"] / 1e3, 1)
+            r["batched_pct_roofline"] = round(100 * r["batched_cold_gbps"] / PEAK_GBPS, 2)
+            m4[name] = r
+            for c in cps:
+                c.free()
+        x4.free()
+        c4.free()
+
     gbps = nbytes / us_gemv / 1e3
     out = {
         "metric": METRIC, "value": round(us_gemv, 3), "unit": "us/GEMV", "n_gpus": 1,
@@ -198,7 +233,7 @@ def main():
                    "protocol": "launches back to back on one stream between two HIP events; value = event time "
                                "/ (steps * gemvs_per_step)"},
         "hbm_gbps": round(gbps, 1), "pct_roofline": round(100 * gbps / PEAK_GBPS, 2),
-        "single_launch": single, "other_encodings": others,
+        "single_launch": single, "other_encodings": others, "config1_m4": m4,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / PEAK_GBPS, 4),
