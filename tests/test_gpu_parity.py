@@ -371,7 +371,7 @@ def test_streams_and_clone():
 
 # ------------------------------------------------------------------ batched launch
 @pytest.mark.parametrize("kind", ["u16", "delta", "i2s"])
-@pytest.mark.parametrize("M,count", [(1, 3), (4, 5), (1, 40)])
+@pytest.mark.parametrize("M,count", [(1, 3), (4, 5), (1, 40), (8, 9), (16, 2)])
 def test_batched_launch_equals_single_launches(kind, M, count):
     K, N, S = 2560, 640, 1536
     W, pos, neg = matrix(K, N, S, dense=True)
