@@ -90,6 +90,28 @@ def test_u16_row_counts(M):
         assert (got == want).all(), split
 
 
+@pytest.mark.parametrize("split", [8, 16, 32, 64, 128, 256])
+def test_multi_row_tiles_every_split(split):
+    """Four- and eight-row tiles (sums on the matrix unit): every lanes-per-column layout of the result tiles."""
+    K, N, S = 2560, 640, 1536
+    say("multi-row tiles, split", split)
+    _, pos, neg = matrix(K, N, S)
+    ws = [sp.Weights.upload_u16(pos, neg, K, split)]
+    if split <= 64:
+        ws.append(sp.Weights.upload_delta(pos, neg, K, split))
+    for M in (4, 8):
+        X = x_i8(300 + M, M, K)
+        want = oracle.sptmm_i8_mt(X, pos, neg, 8)
+        for w in ws:
+            assert (w.matmul(X) == want).all(), (M, w.info["kind"])
+    Xh = oracle.make_x_normal(77, 4, K, np.float16)
+    ref = oracle.sptmm_f64(Xh, pos, neg)
+    for w in ws:
+        check_fp(w.matmul(Xh), ref, S)
+    for w in ws:
+        w.free()
+
+
 @pytest.mark.parametrize("K,N,S,splits", [
     (64, 16, 32, (8, 16)),               # one or two entries per lane: tails only
     (512, 48, 256, (8, 16, 32, 64, 128)),
