@@ -517,7 +517,7 @@ struct ListsBody {
     static constexpr int SLOT = SLOT_OF;
     static constexpr int RING = MT == 8 ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
     static constexpr int XMAX = VAR ? 2 : 0;          // ragged tasks on the straight-line path: full rounds beyond RF a task may have
-    static constexpr int EARLY = 2;                   // rounds requested before the activation tile is complete
+    static constexpr int EARLY = MT >= 4 ? 4 : 2;     // rounds requested before the activation tile is complete (multi-row tiles take longer to stage)
 
     static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, Sums<Act, MT> &acc)
     {
