@@ -273,3 +273,49 @@ def test_i2s_rejects_non_ternary():
     W[3, 5] = 2
     with pytest.raises(sp.SptmmError):
         sp.pack_i2s(W)
+
+
+def test_random_shapes_round_trip_or_are_refused():
+    """300 seeded shapes, valid and invalid alike: every packer either refuses with a status code or
+    round-trips exactly (the same loop runs clean under AddressSanitizer / UBSan on a host-only build)."""
+    rng = np.random.default_rng(7)
+    packed = refused = 0
+    for it in range(300):
+        K = 16 * int(rng.integers(1, 40))
+        N = int(rng.choice([16, 17, 32, 48])) if rng.random() < 0.3 else 16 * int(rng.integers(1, 5))
+        S = int(rng.integers(0, K + 4))
+        if rng.random() < 0.8:
+            S -= S % 2
+        split = int(rng.choice([4, 8, 16, 32, 64, 128, 256, 512, 24]))
+        try:
+            _, pos, neg = sp.generate_ternary(K, N, S)
+        except sp.SptmmError as e:
+            assert e.code == -1
+            refused += 1
+            continue
+        try:
+            buf = sp.pack_u16(pos, neg, K, split)
+            p2, n2 = sp.unpack_u16(buf, K, N, S, split)
+            assert (np.sort(p2, 1) == pos).all() and (np.sort(n2, 1) == neg).all()
+            packed += 1
+        except sp.SptmmError as e:
+            assert e.code == -1
+            refused += 1
+        try:
+            buf, bits = sp.pack_delta(pos, neg, K, split)
+            p2, n2 = sp.unpack_delta(buf, K, N, S, split, bits)
+            assert (p2 == pos).all() and (n2 == neg).all()
+            packed += 1
+        except sp.SptmmError as e:
+            assert e.code == -1
+            refused += 1
+        W = sp.generate_ternary_iid(K, N, it, float(rng.random() * 0.6), float(rng.random() * 0.4))
+        for kind in (sp.KIND_U16, sp.KIND_DELTA):
+            try:
+                buf, meta = sp.pack_ragged(W, kind, split)
+                assert (sp.unpack_ragged(buf, K, N, kind, split, meta["bits"]) == W).all()
+                packed += 1
+            except sp.SptmmError as e:
+                assert e.code == -1
+                refused += 1
+    assert packed > 200 and refused > 200, (packed, refused)
