@@ -451,3 +451,44 @@ def test_batched_launch_rejects_mixed_shapes():
     assert e.value.code == -1
     for o in (a, b, xb, cb):
         o.free()
+
+
+def test_threads_share_one_weights_object():
+    """Four host threads, each with its own stream and buffers, launch on the same weights objects at once."""
+    import threading
+
+    K, N, S = 2560, 640, 1536
+    W, pos, neg = matrix(K, N, S, dense=True)
+    ws = [sp.Weights.upload_u16(pos, neg, K, 32), sp.Weights.upload_delta(pos, neg, K, 16), sp.Weights.upload_i2s(W)]
+    errors = []
+
+    def worker(tid):
+        try:
+            st = sp.Stream()
+            for rep in range(12):
+                M = (1, 4, 8)[(tid + rep) % 3]
+                X = x_i8(4000 + 31 * tid + rep, M, K)
+                want = oracle.sptmm_i8(X, pos, neg)
+                xb = sp.DeviceBuffer.from_numpy(X)
+                cbs = [sp.DeviceBuffer(4 * M * N) for _ in ws]
+                for w, cb in zip(ws, cbs):
+                    w.gemv_i8(xb, M, cb, st)
+                st.sync()
+                for w, cb in zip(ws, cbs):
+                    if not (cb.to_numpy(np.int32, (M, N)) == want).all():
+                        errors.append((tid, rep, w.info["kind"]))
+                for o in [xb] + cbs:
+                    o.free()
+            st.destroy()
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append((tid, repr(e)))
+
+    say("threads: 4 x 12 rounds on shared weights")
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for w in ws:
+        w.free()
+    assert not errors, errors
