@@ -151,7 +151,8 @@ int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weigh
  * other weights object. */
 int sptmm_weights_upload_dense(const int8_t *W_colmajor, int K, int N, int kind, int split_k, sptmm_weights **out);
 /* Second device copy of the same stream (used to rotate over more bytes than
- * the last-level cache holds when timing cold reads). */
+ * the last-level cache holds when timing cold reads).  The copy is complete on
+ * return: a launch on any stream may follow at once. */
 int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out);
 void sptmm_weights_free(sptmm_weights *w);
 /* Weight files, so that the host-side preparation (prepareW_map,
@@ -165,13 +166,21 @@ int sptmm_weights_info(const sptmm_weights *w, sptmm_winfo *out);
 size_t sptmm_weights_bytes(const sptmm_weights *w);
 
 /* C[M][N] = X[M][K] . W, X and C row-major device pointers (main.cu:575,592).
- * Asynchronous on `stream`.
+ * Asynchronous on `stream`.  The device that held the weights at upload must be
+ * the current one (SPTMM_ERR_INVALID otherwise).
  *   sptmm_gemv_i8  int8 activations, exact int32 sums: rowWiseSplit3Small4
  *                  (main.cu:556-594), rowWiseSplit2DeltaSmallAsync2/3
  *                  (main.cu:599-764) or ladder_int8xint2_kernel
  *                  (bitnet_kernels.cuh:75-111), by the kind of `w`.
  *   sptmm_gemv_f16 fp16 activations (raw bits), fp32 sums; u16 and delta kinds.
- *   sptmm_gemv_f32 fp32 activations, fp32 sums; u16 and delta kinds. */
+ *   sptmm_gemv_f32 fp32 activations, fp32 sums; u16 and delta kinds.
+ * Non-finite activations (fp16 / fp32): an Inf or NaN at X[m][k] reaches exactly
+ * the outputs C[m][n] of the columns n whose lists hold row k, as the IEEE sums of
+ * the gathered values give them (Inf, or NaN where +Inf meets -Inf).  Every other
+ * row of the batch and every column that does not gather k is computed as if the
+ * value were not there.  (A workgroup whose activation tile holds a non-finite
+ * value sums on the vector unit instead of the matrix unit -- same result, several
+ * times slower, so that one sequence's overflow never spoils another's.) */
 int sptmm_gemv_i8(const sptmm_weights *w, const int8_t *X_dev, int M, int32_t *C_dev, void *stream);
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X_dev, int M, float *C_dev, void *stream);
 int sptmm_gemv_f32(const sptmm_weights *w, const float *X_dev, int M, float *C_dev, void *stream);
@@ -205,7 +214,7 @@ int sptmm_malloc(void **dev_ptr, size_t bytes);
 int sptmm_free(void *dev_ptr);
 int sptmm_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int sptmm_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes);
-int sptmm_memset(void *dst_dev, int value, size_t bytes);
+int sptmm_memset(void *dst_dev, int value, size_t bytes); /* complete on return, like the two copies */
 int sptmm_stream_create(void **stream);
 int sptmm_stream_destroy(void *stream);
 int sptmm_stream_sync(void *stream);

@@ -92,6 +92,9 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
 {
     if (!w || !X || !C) return fail(SPTMM_ERR_INVALID, "null pointer");
     if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
     GemvArgs a{};
     a.w = w->dev;
     a.X = X;
@@ -250,6 +253,9 @@ int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out)
         c->dev = nullptr;
         hipError_t e = hipMalloc(&c->dev, w->bytes);
         if (e == hipSuccess) e = hipMemcpy(c->dev, w->dev, w->bytes, hipMemcpyDeviceToDevice);
+        // a device-to-device copy need not be complete when hipMemcpy returns, and the streams this library
+        // hands out do not order against the null stream: the copy is finished before the clone is handed back
+        if (e == hipSuccess) e = hipDeviceSynchronize();
         if (e != hipSuccess) {
             if (c->dev) (void)hipFree(c->dev);
             delete c;
@@ -480,6 +486,7 @@ int sptmm_memcpy_d2h(void *d, const void *s, size_t n)
 int sptmm_memset(void *d, int v, size_t n)
 {
     HIP_TRY(hipMemset(d, v, n));
+    HIP_TRY(hipStreamSynchronize(nullptr));  // complete on return, whatever stream the caller launches on next
     return SPTMM_OK;
 }
 int sptmm_stream_create(void **s)

@@ -42,6 +42,7 @@ int make_geometry(int N, int S, int split_k, int max_split, Geometry *g)
     bool ok = false;
     for (int s = 8; s <= max_split; s *= 2) ok |= (s == split_k);
     if (!ok) return fail(SPTMM_ERR_INVALID, "Wrong split size");
+    if (N <= 0 || S <= 0) return fail(SPTMM_ERR_INVALID, "N and S must be positive");
     int half = S / 2;
     if (half % split_k) return fail(SPTMM_ERR_INVALID, "Wrong SPLIT Size: (S/2) %% split_k != 0");
     g->N = N;
@@ -61,6 +62,7 @@ int make_ragged_geometry(int N, int split_k, int max_split, Geometry *g)
     bool ok = false;
     for (int s = 8; s <= max_split; s *= 2) ok |= (s == split_k);
     if (!ok) return fail(SPTMM_ERR_INVALID, "Wrong split size");
+    if (N <= 0) return fail(SPTMM_ERR_INVALID, "N must be positive");
     g->N = N;
     g->half = 0;
     g->split_k = split_k;
@@ -113,29 +115,6 @@ static inline Place place(const Geometry &g, int c, int i, bool contiguous)
     return p;
 }
 
-template <class F>
-static void parallel_columns(int n, F f)
-{
-    // worker threads; the first exception any of them meets is rethrown on the calling thread
-    unsigned hw = std::thread::hardware_concurrency();
-    int nt = (int)std::min<unsigned>(hw ? hw : 1, 16);
-    if (n < 64) nt = 1;
-    std::vector<std::thread> th;
-    std::vector<std::exception_ptr> err(nt);
-    for (int t = 0; t < nt; ++t)
-        th.emplace_back([=, &err] {
-            try {
-                int i0 = (int)((long)n * t / nt), i1 = (int)((long)n * (t + 1) / nt);
-                for (int i = i0; i < i1; ++i) f(i);
-            } catch (...) {
-                err[t] = std::current_exception();
-            }
-        });
-    for (auto &t : th) t.join();
-    for (auto &e : err)
-        if (e) std::rethrow_exception(e);
-}
-
 static inline uint32_t xorshift32(uint32_t &s)
 {
     s ^= s << 13;
@@ -160,7 +139,7 @@ int sptmm_lists_from_dense(const int8_t *W, int K, int N, int S, uint16_t *pos, 
         if (!W || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
         const int half = S / 2;
         std::vector<int> bad(N, 0);
-        parallel_columns(N, [&](int c) {
+        parallel_for(N, [&](int c) {
             const int8_t *w = W + (size_t)c * K;
             int np = 0, nn = 0;
             for (int r = 0; r < K; ++r) {
@@ -188,7 +167,7 @@ int sptmm_generate_ternary(int K, int N, int S, int8_t *W, uint16_t *pos, uint16
         if (int rc = check_shape(K, N, S)) return rc;
         if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
         const int half = S / 2;
-        parallel_columns(N, [&](int c) {
+        parallel_for(N, [&](int c) {
             std::vector<int8_t> local;
             int8_t *w;
             if (W) {
@@ -446,7 +425,7 @@ int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S
         };
         // groups of columns that share half-wavefronts: one column when L >= 32, else 32/L columns
         const int group = g.L >= 32 ? 1 : 32 / g.L;
-        parallel_columns(N / group, [&](int gi) {
+        parallel_for(N / group, [&](int gi) {
             for (int sign = 0; sign < 2; ++sign) {
                 const uint16_t *lists = sign ? neg : pos;
                 if (g.L == 64) {
@@ -501,7 +480,7 @@ int sptmm_unpack_u16(const void *packed, int K, int N, int S, int split_k, uint1
         const int sh = u16_index_shift(K);
         const size_t task_bytes = (size_t)256 * g.n_lane;
         const uint8_t *base = (const uint8_t *)packed;
-        parallel_columns(N, [&](int c) {
+        parallel_for(N, [&](int c) {
             for (int sign = 0; sign < 2; ++sign) {
                 uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
                 for_cells(g, c, [&](int task, int lane, int slot, int i) {
@@ -593,7 +572,7 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
             for (size_t i = 1, e = (size_t)N * g.half; i < e; ++i)
                 if (i % g.n_lane && l[i] <= l[i - 1]) return fail(SPTMM_ERR_INVALID, "row lists must be strictly ascending");
         }
-        parallel_columns(g.tasks, [&](int t) {
+        parallel_for(g.tasks, [&](int t) {
             std::vector<uint16_t> rows[2][64];
             for (int sign = 0; sign < 2; ++sign)
                 for (int lane = 0; lane < 64; ++lane) {
@@ -606,7 +585,7 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
             if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d: a gap does not fit 8 bits (signed)", c);
         return SPTMM_OK;
     }
-    parallel_columns(N, [&](int c) {
+    parallel_for(N, [&](int c) {
         for (int sign = 0; sign < 2; ++sign) {
             uint16_t *lst = (sign ? neg : pos) + (size_t)c * g.half;
             int run = 0;
@@ -645,9 +624,13 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
 int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out)
 {
     return guarded([&]() -> int {
-        if (pos && neg)
-            for (size_t i = 0, n = (size_t)N * (S / 2); i < n; ++i)
-                if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
+        // shape first: the scan below trusts N and S
+        if (int rc = check_shape(K, N, S)) return rc;
+        Geometry g;
+        if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
+        if (!out || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+        for (size_t i = 0, n = (size_t)N * g.half; i < n; ++i)
+            if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
         return delta_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k, bits);
     });
 }
@@ -694,7 +677,7 @@ int sptmm_pack_i2s(const int8_t *W, int K, int N, void *out)
         const int Kp = i2s_padded_k(K);
         uint32_t *o = (uint32_t *)out;
         std::vector<int> bad(N, 0);
-        parallel_columns(N, [&](int c) {
+        parallel_for(N, [&](int c) {
             for (int g16 = 0; g16 < Kp / 16; ++g16) {
                 int8_t w16[16] = {0};
                 if (g16 * 16 < K) {

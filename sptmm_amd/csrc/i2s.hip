@@ -5,25 +5,11 @@
 #include <atomic>
 
 #include "internal.hpp"
+#include "lanes.hpp"
 
 namespace sptmm {
 
 typedef unsigned int u32;
-
-template <int CTRL> __device__ __forceinline__ int dpp(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
-__device__ __forceinline__ int swz16(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401f); }  // lane ^ 16
-
-// Sum over groups of 2^logL consecutive lanes (logL >= 2); every lane of a group ends with the group's total.
-__device__ __forceinline__ int lanes_sum(int v, int logL)
-{
-    v += dpp<0xB1>(v);                   // quad_perm [1,0,3,2]
-    v += dpp<0x4E>(v);                   // quad_perm [2,3,0,1]
-    if (logL >= 3) v += dpp<0x141>(v);   // row_half_mirror
-    if (logL >= 4) v += dpp<0x140>(v);   // row_mirror
-    if (logL >= 5) v += swz16(v);
-    if (logL >= 6) v += __shfl_xor(v, 32, 64);
-    return v;
-}
 
 // ------------------------------------------------------------------- i2s GEMV
 struct I2sParams {

@@ -5,7 +5,9 @@
 #include <cstddef>
 #include <cstdint>
 #include <exception>
+#include <algorithm>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "../../include/sptmm.h"
@@ -26,6 +28,29 @@ template <class F> int guarded(F body) noexcept
     } catch (...) {
         return fail(SPTMM_ERR_INVALID, "unexpected exception");
     }
+}
+
+// f(i) for i in [0, n) on up to 16 worker threads (one below 64 items); the first exception any
+// worker meets is rethrown on the calling thread.
+template <class F> void parallel_for(int n, F f)
+{
+    unsigned hw = std::thread::hardware_concurrency();
+    int nt = (int)std::min<unsigned>(hw ? hw : 1, 16);
+    if (n < 64) nt = 1;
+    std::vector<std::thread> th;
+    std::vector<std::exception_ptr> err(nt);
+    for (int t = 0; t < nt; ++t)
+        th.emplace_back([=, &err] {
+            try {
+                int i0 = (int)((long)n * t / nt), i1 = (int)((long)n * (t + 1) / nt);
+                for (int i = i0; i < i1; ++i) f(i);
+            } catch (...) {
+                err[t] = std::current_exception();
+            }
+        });
+    for (auto &t : th) t.join();
+    for (auto &e : err)
+        if (e) std::rethrow_exception(e);
 }
 
 // ---- geometry of the wave64 streams --------------------------------------

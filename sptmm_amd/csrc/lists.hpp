@@ -11,6 +11,7 @@
 #include <type_traits>
 
 #include "internal.hpp"
+#include "lanes.hpp"
 
 namespace sptmm {
 
@@ -49,11 +50,20 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 // (-1 for the minus list) that routes every byte to the int32 of its (lane, row) in the 16x16
 // result.  Nothing is contracted -- each output sums one lane's own bytes of one row -- the
 // instruction is used as 256 byte-to-int32 adders, on a unit this kernel otherwise leaves idle.
-template <typename Act, int MT> struct Sums {
+//
+// PLAIN = true: fp16 rows summed on the VALU whatever MT (one convert and one add per entry and
+// row).  The matrix-unit sums multiply every byte of an operand row with 0 or +-1, so one Inf or
+// NaN among the gathered values turns the sums of the other rows and of the three partner lanes
+// into NaN (0 x Inf); a workgroup whose tile holds a non-finite value therefore sums this way.
+template <typename Act, int MT, bool PLAIN = false> struct Sums {
     typedef typename Acc<Act>::type A;
+    typedef Act act_type;
+    static constexpr int ROWS = MT;
+    static constexpr int SLOT = slot_bytes<Act, MT>();
+    static_assert(!PLAIN || sizeof(Act) == 2, "only fp16 tiles have a VALU twin");
     static constexpr bool MX = sizeof(Act) == 1 && MT > 1;  // sums on the matrix unit
-    static constexpr bool MXF = sizeof(Act) == 2 && MT > 1; // the same for fp16 rows (MT = 4): v_mfma_f32_16x16x32_f16,
-                                                            // two entries x four rows per operand, selector of 0 / +-1.0
+    static constexpr bool MXF = sizeof(Act) == 2 && MT > 1 && !PLAIN;  // the same for fp16 rows (MT = 4): v_mfma_f32_16x16x32_f16,
+                                                                       // two entries x four rows per operand, selector of 0 / +-1.0
     static constexpr int NW = MX ? MT / 4 : 1;              // dwords per gathered slot (int8)
     static constexpr int ND = MX ? MT / 4 : 1;              // result tiles
     v4i D[ND], Bp[ND], Bn[ND];                              // MX: 16x16 int32 result tiles and the +1 / -1 selectors
@@ -201,11 +211,10 @@ template <int B> __device__ __forceinline__ void add_signed_byte(u32 &run, u32 d
 // the byte offset of the row's slot in the tile with 16-bit gaps.  fetch() turns
 // the low NBYTES of `d` into tile reads; the adds follow separately so that the
 // compiler is free to keep several reads in flight.
-template <typename Act, int MT, int MODE, bool PRE, int NBYTES>
-__device__ __forceinline__ void fetch(const unsigned char *lds, u32 d, u32 &run, typename Sums<Act, MT>::Raw *r)
+template <class S, int MODE, bool PRE, int NBYTES>
+__device__ __forceinline__ void fetch(const unsigned char *lds, u32 d, u32 &run, typename S::Raw *r)
 {
-    typedef Sums<Act, MT> S;
-    constexpr int SH = ilog2(slot_bytes<Act, MT>());
+    constexpr int SH = ilog2(S::SLOT);
     if constexpr (Flavour<MODE>::GAP8) {
         add_signed_byte<0>(run, d);
         r[0] = S::load(lds, run << SH);
@@ -233,24 +242,24 @@ __device__ __forceinline__ void fetch(const unsigned char *lds, u32 d, u32 &run,
     }
 }
 
-template <typename Act, int MT, int MODE, bool PRE, bool NEG, int NBYTES>
-__device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &run, Sums<Act, MT> &acc)
+template <class S, int MODE, bool PRE, bool NEG, int NBYTES>
+__device__ __forceinline__ void consume(const unsigned char *lds, u32 d, u32 &run, S &acc)
 {
     constexpr int NE = NBYTES / Flavour<MODE>::ESZ;
-    typename Sums<Act, MT>::Raw r[NE];
-    fetch<Act, MT, MODE, PRE, NBYTES>(lds, d, run, r);
+    typename S::Raw r[NE];
+    fetch<S, MODE, PRE, NBYTES>(lds, d, run, r);
     acc.template accum_n<NEG, NE>(r);
 }
 
-template <typename Act, int MT, int MODE, bool PRE, bool NEG>
-__device__ __forceinline__ void consume16(const unsigned char *lds, const uint4 &v, u32 &run, Sums<Act, MT> &acc)
+template <class S, int MODE, bool PRE, bool NEG>
+__device__ __forceinline__ void consume16(const unsigned char *lds, const uint4 &v, u32 &run, S &acc)
 {
     constexpr int NE = 4 / Flavour<MODE>::ESZ;  // entries per dword
-    typename Sums<Act, MT>::Raw r[4 * NE];
-    fetch<Act, MT, MODE, PRE, 4>(lds, v.x, run, r);
-    fetch<Act, MT, MODE, PRE, 4>(lds, v.y, run, r + NE);
-    fetch<Act, MT, MODE, PRE, 4>(lds, v.z, run, r + 2 * NE);
-    fetch<Act, MT, MODE, PRE, 4>(lds, v.w, run, r + 3 * NE);
+    typename S::Raw r[4 * NE];
+    fetch<S, MODE, PRE, 4>(lds, v.x, run, r);
+    fetch<S, MODE, PRE, 4>(lds, v.y, run, r + NE);
+    fetch<S, MODE, PRE, 4>(lds, v.z, run, r + 2 * NE);
+    fetch<S, MODE, PRE, 4>(lds, v.w, run, r + 3 * NE);
     acc.template accum_n<NEG, 4 * NE>(r);
 }
 
@@ -287,6 +296,39 @@ __device__ __forceinline__ void swap_if(bool c, u32 &a, u32 &b)
 __device__ __forceinline__ u32 comp(const uint4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
 __device__ __forceinline__ u32 f2u(float f) { return __builtin_bit_cast(u32, f); }
 __device__ __forceinline__ float h2f(u32 d, int hi) { return (float)__builtin_bit_cast(_Float16, (unsigned short)(hi ? d >> 16 : d & 0xffffu)); }
+
+// Running maxima of |x| as 16-bit patterns, two per register: for fp16 and bf16 alike, clearing
+// the sign bit leaves patterns that order like the magnitudes they encode (Inf and NaN on top).
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 pk_absmax16(u32 mx, u32 d)
+{
+    return __builtin_bit_cast(u32, __builtin_elementwise_max(__builtin_bit_cast(u16x2, mx), __builtin_bit_cast(u16x2, d & 0x7fff7fffu)));
+}
+__device__ __forceinline__ u32 pk_absmax16(u32 mx, const uint4 &v) { return pk_absmax16(pk_absmax16(pk_absmax16(pk_absmax16(mx, v.x), v.y), v.z), v.w); }
+// either half holds the pattern of an fp16 Inf or NaN
+__device__ __forceinline__ bool pk_nonfinite16(u32 mx) { return (mx & 0xffffu) >= 0x7c00u || (mx >> 16) >= 0x7c00u; }
+
+// Byte offset, inside a task's rounds, of entry j of `lane` for `sign` (0 = +1 list): full rounds of
+// 16 bytes per lane and sign, then at most one round each of 8, 4, 2 (and 1) bytes per lane.
+template <int ESZ> __device__ __forceinline__ u32 entry_offset(int n_lane, int sign, int lane, int j)
+{
+    constexpr int E16 = 16 / ESZ;
+    const int full = n_lane / E16;
+    if (j < full * E16) return (u32)(j / E16) * 2048u + (u32)sign * 1024u + (u32)lane * 16u + (u32)(j % E16) * ESZ;
+    u32 base = (u32)full * 2048u;
+    const int rem = n_lane - full * E16;
+    int first = full * E16;
+#pragma unroll
+    for (int w = 8; w >= ESZ; w /= 2) {
+        const int cnt = w / ESZ;
+        if (rem & cnt) {
+            if (j < first + cnt) return base + (u32)sign * 64u * w + (u32)lane * w + (u32)(j - first) * ESZ;
+            first += cnt;
+            base += 128u * w;
+        }
+    }
+    return base;
+}
 
 // Staging of the activation tile, in items of 16 consecutive k for all MT rows.
 // load() pulls an item into registers (rows past M read as zero); store()
@@ -378,28 +420,6 @@ template <typename Act, int MT> struct Stager {
     }
 };
 
-template <int CTRL> __device__ __forceinline__ int dpp(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
-template <int CTRL> __device__ __forceinline__ float dpp(float v) { return __builtin_bit_cast(float, dpp<CTRL>(__builtin_bit_cast(int, v))); }
-__device__ __forceinline__ int swz16(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401f); }  // lane ^ 16
-__device__ __forceinline__ int swz8(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x201f); }   // lane ^ 8
-__device__ __forceinline__ int swz4(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x101f); }   // lane ^ 4
-__device__ __forceinline__ float swz16(float v) { return __builtin_bit_cast(float, swz16(__builtin_bit_cast(int, v))); }
-__device__ __forceinline__ float swz8(float v) { return __builtin_bit_cast(float, swz8(__builtin_bit_cast(int, v))); }
-__device__ __forceinline__ float swz4(float v) { return __builtin_bit_cast(float, swz4(__builtin_bit_cast(int, v))); }
-
-// Sum over groups of 2^logL consecutive lanes (logL >= 2); every lane of a group ends with the group's total.
-template <typename T>
-__device__ __forceinline__ T lanes_sum(T v, int logL)
-{
-    v += dpp<0xB1>(v);                   // quad_perm [1,0,3,2]
-    v += dpp<0x4E>(v);                   // quad_perm [2,3,0,1]
-    if (logL >= 3) v += dpp<0x141>(v);   // row_half_mirror
-    if (logL >= 4) v += dpp<0x140>(v);   // row_mirror
-    if (logL >= 5) v += swz16(v);
-    if (logL >= 6) v += __shfl_xor(v, 32, 64);
-    return v;
-}
-
 struct ListParams {
     const uint8_t *w;
     const void *X;
@@ -418,6 +438,13 @@ constexpr int LISTS_MAX_WAVES = 8;  // 512 threads: two wavefronts per SIMD, 256
 // room for one workgroup per CU only, so that workgroup has to bring the wavefronts that fill
 // the four SIMDs itself: 1024 threads, four wavefronts per SIMD, 128 VGPRs each.
 template <typename Act, int MT, bool QUANT> constexpr int lists_max_waves() { return sizeof(Act) == 1 && MT >= 4 && !QUANT ? 16 : LISTS_MAX_WAVES; }
+
+// LDS a workgroup of `waves` wavefronts keeps behind the activation tile: the per-wavefront sums of
+// columns that span wavefronts, and for fp16 tiles summed on the matrix unit one flag per wavefront.
+template <typename Act, int MT> constexpr size_t lists_behind_tile(int waves)
+{
+    return (size_t)waves * MT * 4 + (sizeof(Act) == 2 && MT > 1 ? (size_t)waves * 4 : 0);
+}
 
 // One round of a task's stream: 16 bytes per lane of the +1 list and of the -1 list.
 struct Round {
@@ -444,7 +471,6 @@ __device__ __forceinline__ Round load_round(const uint4 *wp, int r)
 // hand back floats.  Item = 16 consecutive k of all MT rows, as in Stager.
 template <int MT> struct Quantiser {
     static constexpr int HOLD = MT <= 4 ? 2 : 0;  // items a thread keeps in registers between the two passes (the rest is read twice)
-    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 
     // 2 x 16 bytes per row: the item's 16 values of row m0 + m (rows past M read as zero)
     static __device__ __forceinline__ void load(const unsigned short *X, int M, int K, int m0, int item, uint4 (&r)[2 * MT])
@@ -456,17 +482,11 @@ template <int MT> struct Quantiser {
                 r[2 * m + j] = (m0 + m < M) ? reinterpret_cast<const uint4 *>(X + (size_t)(m0 + m) * K)[(size_t)item * 2 + j]
                                             : make_uint4(0, 0, 0, 0);
     }
-    // Running maxima of |x| as bit patterns, two per register: for fp16 and bf16 alike, clearing
-    // the sign bit leaves patterns that order like the magnitudes they encode.
+    // running maxima of |x| per row, as packed bit patterns
     static __device__ __forceinline__ void absmax(const uint4 (&r)[2 * MT], u32 (&mx)[MT])
     {
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const u32 d = comp(r[2 * m + c / 4], c % 4) & 0x7fff7fffu;
-                mx[m] = __builtin_bit_cast(u32, __builtin_elementwise_max(__builtin_bit_cast(u16x2, mx[m]), __builtin_bit_cast(u16x2, d)));
-            }
+        for (int m = 0; m < MT; ++m) mx[m] = pk_absmax16(pk_absmax16(mx[m], r[2 * m]), r[2 * m + 1]);
     }
     static __device__ __forceinline__ float magnitude(u32 packed, int kind)
     {
@@ -521,10 +541,64 @@ struct ListsBody {
 
     static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, Sums<Act, MT> &acc)
     {
-        consume16<Act, MT, MODE, PRE, false>(smem, x.p, runp, acc);
-        consume16<Act, MT, MODE, PRE, true>(smem, x.q, runq, acc);
+        consume16<Sums<Act, MT>, MODE, PRE, false>(smem, x.p, runp, acc);
+        consume16<Sums<Act, MT>, MODE, PRE, true>(smem, x.q, runq, acc);
         acc.pin();  // (and the running rows)
         if constexpr (GAPS) asm volatile("" : "+v"(runp), "+v"(runq));
+    }
+
+    // fp16 tiles summed on the matrix unit have a VALU twin for workgroups whose tile holds an Inf or NaN
+    static constexpr bool TWIN = Sums<Act, MT>::MXF;
+    typedef Sums<Act, MT, TWIN> Plain;
+
+    // One task summed on the VALU with a single round in flight (the twin's path: rare, so small rather than fast).
+    static __device__ __forceinline__ void walk_plain(const unsigned char *smem, const uint8_t *tb, int lane, int n_lane, u32 runp, u32 runq,
+                                                      Plain &acc)
+    {
+        const uint4 *wp = reinterpret_cast<const uint4 *>(tb + HDR) + lane;
+        const int R = n_lane / E16;
+#pragma unroll 1
+        for (int r = 0; r < R; ++r) {
+            const Round x = load_round(wp, r);
+            consume16<Plain, MODE, PRE, false>(smem, x.p, runp, acc);
+            consume16<Plain, MODE, PRE, true>(smem, x.q, runq, acc);
+        }
+#pragma unroll 1
+        for (int j = R * E16; j < n_lane; ++j) {
+            const uint8_t *ep = tb + HDR + entry_offset<ESZ>(n_lane, 0, lane, j), *eq = tb + HDR + entry_offset<ESZ>(n_lane, 1, lane, j);
+            const u32 fp = ESZ == 1 ? (u32)*ep : (u32)*reinterpret_cast<const unsigned short *>(ep);
+            const u32 fq = ESZ == 1 ? (u32)*eq : (u32)*reinterpret_cast<const unsigned short *>(eq);
+            consume<Plain, MODE, PRE, false, ESZ>(smem, fp, runp, acc);
+            consume<Plain, MODE, PRE, true, ESZ>(smem, fq, runq, acc);
+        }
+    }
+
+    // Per-lane sums of a task -> column totals: folded over the L lanes of a column, then written (one
+    // wavefront per column or less) or left in `part` for the second pass (columns that span wavefronts).
+    static __device__ __forceinline__ void store_lane_sums(const ListParams &p, A (&v)[MT], A *part, const float (&back)[MT], bool active,
+                                                           int task, int lane, int wave, int m0)
+    {
+        A *C = reinterpret_cast<A *>(p.C);
+        float *Cf = reinterpret_cast<float *>(p.C);  // quantising kernels: acc / s * w_scale
+        const int L = 1 << p.logL;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) v[m] = lanes_sum(v[m], p.logL);
+        if (p.W == 1) {
+            if (active && (lane & (L - 1)) == 0) {
+                const int col = (task << (6 - p.logL)) + (lane >> p.logL);
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    if (m0 + m < p.M) {
+                        if constexpr (QUANT)
+                            Cf[(size_t)(m0 + m) * p.N + col] = (float)v[m] * back[m] * p.w_scale;
+                        else
+                            C[(size_t)(m0 + m) * p.N + col] = v[m];
+                    }
+            }
+        } else if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) part[wave * MT + m] = v[m];
+        }
     }
 
     // RF > 0: the task has exactly RF full rounds (ragged: RF to RF + XMAX) and
@@ -572,6 +646,7 @@ struct ListsBody {
                 St::load(X, p.M, p.K, m0, item < items ? item : items - 1, xr[i]);
             }
         }
+        u32 xmax = 0u;  // TWIN: largest |x| pattern this thread has staged
         // ragged: the first task's entry count travels with the activation loads, so it is there
         // long before the tile is; every later count is asked for one task ahead
         int n_ahead = p.n_lane;
@@ -636,6 +711,12 @@ struct ListsBody {
 #pragma unroll
             for (int i = 0; i < St::XI; ++i)
                 if (tid + i * nt < items) St::store(smem, tid + i * nt, xr[i]);
+            if constexpr (TWIN) {
+#pragma unroll
+                for (int i = 0; i < St::XI; ++i)
+#pragma unroll
+                    for (int j = 0; j < St::NLOAD; ++j) xmax = pk_absmax16(xmax, xr[i][j]);
+            }
         }
         if constexpr (RF > EARLY) {
             const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
@@ -653,19 +734,34 @@ struct ListsBody {
                 uint4 r[St::NLOAD];
                 St::load(X, p.M, p.K, m0, item, r);
                 St::store(smem, item, r);
+                if constexpr (TWIN) {
+#pragma unroll
+                    for (int j = 0; j < St::NLOAD; ++j) xmax = pk_absmax16(xmax, r[j]);
+                }
             }
         }
         // rows K.. read as zero
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
             reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = 0u;
+        // TWIN: one flag per wavefront behind the per-wavefront sums, folded by every thread after the barrier
+        u32 *nf_flags = reinterpret_cast<u32 *>(part + waves * MT);
+        if constexpr (TWIN) {
+            const bool any = __builtin_amdgcn_ballot_w64(pk_nonfinite16(xmax)) != 0;
+            if (lane == 0) nf_flags[wave] = any ? 1u : 0u;
+        }
         __syncthreads();
+        bool plain = false;  // workgroup-uniform
+        if constexpr (TWIN) {
+            u32 f = 0u;
+            for (int w = 0; w < waves; ++w) f |= nf_flags[w];
+            plain = __builtin_amdgcn_readfirstlane(f) != 0u;
+        }
 
         A *C = reinterpret_cast<A *>(p.C);
         float *Cf = reinterpret_cast<float *>(p.C);  // quantising kernels: acc / s * w_scale
         float back[MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m) back[m] = QUANT ? qinv[m] : 0.f;
-        const int L = 1 << p.logL;
         for (int it = 0; it < p.iters; ++it, task += task_step) {
             const bool active = task < p.tasks;
             const uint8_t *tb = tasks_base + (size_t)(active ? task : 0) * task_bytes;
@@ -683,6 +779,12 @@ struct ListsBody {
                 n_ahead = counts[nxt < p.tasks ? nxt : 0];
             }
             const int R = n_lane / E16, rem = n_lane - R * E16;
+            if (TWIN && plain) {
+                Plain pacc;
+                pacc.init();
+                walk_plain(smem, tb, lane, n_lane, runp, runq, pacc);
+                store_lane_sums(p, pacc.acc, part, back, active, task, lane, wave, m0);
+            } else {
             Sums<Act, MT> acc;
             acc.init();
 
@@ -770,23 +872,23 @@ struct ListsBody {
             }
             if (rem) {
                 if (rem & (8 / ESZ)) {
-                    consume<Act, MT, MODE, PRE, false, 4>(smem, t8p.x, runp, acc);
-                    consume<Act, MT, MODE, PRE, false, 4>(smem, t8p.y, runp, acc);
-                    consume<Act, MT, MODE, PRE, true, 4>(smem, t8q.x, runq, acc);
-                    consume<Act, MT, MODE, PRE, true, 4>(smem, t8q.y, runq, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, false, 4>(smem, t8p.x, runp, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, false, 4>(smem, t8p.y, runp, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, true, 4>(smem, t8q.x, runq, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, true, 4>(smem, t8q.y, runq, acc);
                 }
                 if (rem & (4 / ESZ)) {
-                    consume<Act, MT, MODE, PRE, false, 4>(smem, t4p, runp, acc);
-                    consume<Act, MT, MODE, PRE, true, 4>(smem, t4q, runq, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, false, 4>(smem, t4p, runp, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, true, 4>(smem, t4q, runq, acc);
                 }
                 if (rem & (2 / ESZ)) {
-                    consume<Act, MT, MODE, PRE, false, 2>(smem, t2p, runp, acc);
-                    consume<Act, MT, MODE, PRE, true, 2>(smem, t2q, runq, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, false, 2>(smem, t2p, runp, acc);
+                    consume<Sums<Act, MT>, MODE, PRE, true, 2>(smem, t2q, runq, acc);
                 }
                 if constexpr (ESZ == 1) {
                     if (rem & 1) {
-                        consume<Act, MT, MODE, PRE, false, 1>(smem, t1p, runp, acc);
-                        consume<Act, MT, MODE, PRE, true, 1>(smem, t1q, runq, acc);
+                        consume<Sums<Act, MT>, MODE, PRE, false, 1>(smem, t1p, runp, acc);
+                        consume<Sums<Act, MT>, MODE, PRE, true, 1>(smem, t1q, runq, acc);
                     }
                 }
             }
@@ -841,25 +943,9 @@ struct ListsBody {
                     part[wave * MT + lane] = t[0];
                 }
             } else {
-#pragma unroll
-                for (int m = 0; m < MT; ++m) acc.acc[m] = lanes_sum(acc.acc[m], p.logL);
-                if (p.W == 1) {
-                    if (active && (lane & (L - 1)) == 0) {
-                        const int col = (task << (6 - p.logL)) + (lane >> p.logL);
-#pragma unroll
-                        for (int m = 0; m < MT; ++m)
-                            if (m0 + m < p.M) {
-                                if constexpr (QUANT)
-                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)acc.acc[m] * back[m] * p.w_scale;
-                                else
-                                    C[(size_t)(m0 + m) * p.N + col] = acc.acc[m];
-                            }
-                    }
-                } else if (lane == 0) {
-#pragma unroll
-                    for (int m = 0; m < MT; ++m) part[wave * MT + m] = acc.acc[m];
-                }
+                store_lane_sums(p, acc.acc, part, back, active, task, lane, wave, m0);
             }
+            }  // matrix-unit / plain sums
             if (p.W != 1) {
                 // second pass: the W wavefronts of a column meet in a small LDS buffer
                 __syncthreads();
@@ -948,7 +1034,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(a.K + 64) * SLOT;
     // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better
-    const bool roomy = a.batch && 2 * (tile + (size_t)LISTS_MAX_WAVES * MT * 4) <= (size_t)a.lds_limit;
+    const bool roomy = a.batch && 2 * (tile + lists_behind_tile<Act, MT>(LISTS_MAX_WAVES)) <= (size_t)a.lds_limit;
     const int max_waves = a.quant || roomy ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>();
     static std::atomic<int> vgprs{0};  // of the single-GEMV kernel of this instantiation
     int regs = vgprs.load(std::memory_order_relaxed);
@@ -968,7 +1054,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         if (tune_wgs > 0 && g != tune_wgs) continue;
         for (int w = a.W; w <= max_waves; w += a.W) {
             if (g > 1 && g * w > 4 * waves_per_simd) continue;  // the register file of the CU's 4 SIMDs
-            if (g > 1 && g * (tile + (size_t)w * MT * 4) > (size_t)a.lds_limit) continue;
+            if (g > 1 && g * (tile + lists_behind_tile<Act, MT>(w)) > (size_t)a.lds_limit) continue;
             const int blocks = (a.tasks + w - 1) / w;
             const int grid = blocks < cus * g ? blocks : cus * g;
             const int iters = (blocks + grid - 1) / grid;
@@ -996,7 +1082,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
                  a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale};
-    size_t lds = (size_t)(a.K + 64) * SLOT + (size_t)wpb * MT * sizeof(typename Acc<Act>::type);
+    size_t lds = (size_t)(a.K + 64) * SLOT + lists_behind_tile<Act, MT>(wpb);
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     if (a.batch) {
@@ -1082,11 +1168,18 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
 template <typename Act, int MODE, bool PRE, bool VAR>
 static int launch_lists_m(const GemvArgs &a, hipStream_t st)
 {
-    const size_t lim = (size_t)a.lds_limit - 256;
+    // a tile of `mt` rows fits when it leaves room for what the largest workgroup keeps behind it: the
+    // per-wavefront sums, and for quantising launches the row maxima and scales as well
+    auto fits = [&](size_t slot, int mt, size_t behind) {
+        const size_t extra = a.quant ? (size_t)(2 * LISTS_MAX_WAVES + 1) * mt * 4 : behind;
+        return (size_t)(a.K + 64) * slot + extra <= (size_t)a.lds_limit;
+    };
     if constexpr (sizeof(Act) == 1) {
-        if (a.M >= 5 && (size_t)(a.K + 64) * slot_bytes<Act, 8>() <= lim) return launch_lists_t<Act, 8, MODE, PRE, VAR>(a, st);
+        if (a.M >= 5 && fits(slot_bytes<Act, 8>(), 8, lists_behind_tile<Act, 8>(lists_max_waves<Act, 8, false>())))
+            return launch_lists_t<Act, 8, MODE, PRE, VAR>(a, st);
     }
-    if (a.M >= 2 && (size_t)(a.K + 64) * slot_bytes<Act, 4>() <= lim) return launch_lists_t<Act, 4, MODE, PRE, VAR>(a, st);
+    if (a.M >= 2 && fits(slot_bytes<Act, 4>(), 4, lists_behind_tile<Act, 4>(lists_max_waves<Act, 4, false>())))
+        return launch_lists_t<Act, 4, MODE, PRE, VAR>(a, st);
     return launch_lists_t<Act, 1, MODE, PRE, VAR>(a, st);
 }
 

@@ -24,29 +24,6 @@ namespace sptmm {
 
 namespace {
 
-template <class F>
-void parallel_for(int n, F f)
-{
-    // worker threads; the first exception any of them meets is rethrown on the calling thread
-    unsigned hw = std::thread::hardware_concurrency();
-    int nt = (int)std::min<unsigned>(hw ? hw : 1, 16);
-    if (n < 64) nt = 1;
-    std::vector<std::thread> th;
-    std::vector<std::exception_ptr> err(nt);
-    for (int t = 0; t < nt; ++t)
-        th.emplace_back([=, &err] {
-            try {
-                int i0 = (int)((long)n * t / nt), i1 = (int)((long)n * (t + 1) / nt);
-                for (int i = i0; i < i1; ++i) f(i);
-            } catch (...) {
-                err[t] = std::current_exception();
-            }
-        });
-    for (auto &t : th) t.join();
-    for (auto &e : err)
-        if (e) std::rethrow_exception(e);
-}
-
 struct RaggedPlan {
     Geometry g;
     int K = 0, kind = 0, bits = 0, esz = 2, hdr = 0, shift = 0;
@@ -298,14 +275,20 @@ int sptmm_dense_from_i2s_words(const uint32_t *words, int K, int N, int8_t *W)
 size_t sptmm_pack_ragged_bytes(const int8_t *W, int K, int N, int kind, int split_k, int *bits, size_t *read_bytes, int *n_min,
                                int *n_max, uint64_t *nnz)
 {
-    RaggedPlan pl;
-    if (ragged_plan(W, K, N, kind, split_k, bits ? *bits : 0, &pl)) return 0;
-    if (bits) *bits = pl.bits;
-    if (read_bytes) *read_bytes = pl.read_bytes;
-    if (n_min) *n_min = pl.n_min;
-    if (n_max) *n_max = pl.n_max;
-    if (nnz) *nnz = pl.nnz;
-    return pl.counts_bytes + pl.stride * pl.g.tasks;
+    // the planner allocates and starts threads: nothing it throws may cross the C ABI (0 = failure, message set)
+    size_t total = 0;
+    const int rc = guarded([&]() -> int {
+        RaggedPlan pl;
+        if (int prc = ragged_plan(W, K, N, kind, split_k, bits ? *bits : 0, &pl)) return prc;
+        if (bits) *bits = pl.bits;
+        if (read_bytes) *read_bytes = pl.read_bytes;
+        if (n_min) *n_min = pl.n_min;
+        if (n_max) *n_max = pl.n_max;
+        if (nnz) *nnz = pl.nnz;
+        total = pl.counts_bytes + pl.stride * pl.g.tasks;
+        return SPTMM_OK;
+    });
+    return rc == SPTMM_OK ? total : 0;
 }
 
 int sptmm_pack_ragged(const int8_t *W, int K, int N, int kind, int split_k, int bits, void *out)

@@ -319,3 +319,36 @@ def test_random_shapes_round_trip_or_are_refused():
                 assert e.code == -1
                 refused += 1
     assert packed > 200 and refused > 200, (packed, refused)
+
+
+def test_non_positive_shapes_are_refused_before_anything_is_read():
+    """Negative or zero K, N, S reach every packer with buffers sized for a small valid shape: each call must
+    return a status code without touching memory beyond them (the same loop runs under AddressSanitizer)."""
+    L = sp.lib()
+    pos = np.zeros((16, 16), np.uint16)
+    neg = np.ones((16, 16), np.uint16)
+    W = np.zeros((16, 64), np.int8)
+    out = np.zeros(1 << 16, np.uint8)
+    P = lambda a: a.ctypes.data
+    import ctypes as C
+
+    for K, N, S in [(64, -16, 32), (64, 16, -32), (-64, 16, 32), (0, 16, 32), (64, 0, 32), (64, 16, 0), (64, -16, -32),
+                    (-64, -16, -32), (64, 16, -2), (64, -1, 32)]:
+        for split in (8, 16, 64):
+            assert L.sptmm_pack_u16(C.c_void_p(P(pos)), C.c_void_p(P(neg)), K, N, S, split, C.c_void_p(P(out))) == -1
+            assert L.sptmm_unpack_u16(C.c_void_p(P(out)), K, N, S, split, C.c_void_p(P(pos)), C.c_void_p(P(neg))) == -1
+            for bits in (8, 16):
+                assert L.sptmm_pack_delta(C.c_void_p(P(pos)), C.c_void_p(P(neg)), K, N, S, split, bits, C.c_void_p(P(out))) == -1
+                assert L.sptmm_unpack_delta(C.c_void_p(P(out)), K, N, S, split, bits, C.c_void_p(P(pos)), C.c_void_p(P(neg))) == -1
+                assert N > 0 and S > 0 or L.sptmm_pack_delta_bytes(N, S, split, bits) == 0  # (takes no K)
+            if N <= 0 or S <= 0:
+                assert L.sptmm_delta_bits(C.c_void_p(P(pos)), C.c_void_p(P(neg)), N, S, split) == -1
+                assert L.sptmm_pack_u16_bytes(N, S, split) == 0
+            assert L.sptmm_generate_ternary(K, N, S, None, C.c_void_p(P(pos)), C.c_void_p(P(neg))) == -1
+            assert L.sptmm_lists_from_dense(C.c_void_p(P(W)), K, N, S, C.c_void_p(P(pos)), C.c_void_p(P(neg))) == -1
+    for K, N in [(-64, 16), (64, -16), (0, 16), (64, 0), (-16, -16)]:
+        for kind in (sp.KIND_U16, sp.KIND_DELTA):
+            assert L.sptmm_pack_ragged_bytes(C.c_void_p(P(W)), K, N, kind, 32, None, None, None, None, None) == 0
+            assert L.sptmm_pack_ragged(C.c_void_p(P(W)), K, N, kind, 32, 8, C.c_void_p(P(out))) == -1
+        assert L.sptmm_pack_i2s_bytes(K, N) == 0
+        assert L.sptmm_pack_i2s(C.c_void_p(P(W)), K, N, C.c_void_p(P(out))) == -1

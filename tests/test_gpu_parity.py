@@ -51,6 +51,8 @@ def x_i8(seed, M, K):
 
 
 def check_fp(got, ref, S):
+    if got.size == 0:
+        return
     scale = np.maximum(np.abs(ref), np.sqrt(S))
     err = np.abs(got.astype(np.float64) - ref) / scale
     assert err.max() <= REL_TOL, "max rel err %.3e" % err.max()
@@ -268,6 +270,63 @@ def test_u16_float_activations(dtype, M):
         check_fp(got, ref, S)
 
 
+def finite_columns(pos, neg, k):
+    """Columns whose lists do not hold row k."""
+    return ~((pos == k).any(axis=1) | (neg == k).any(axis=1))
+
+
+@pytest.mark.parametrize("kind,split", [("u16", 8), ("u16", 16), ("u16", 32), ("u16", 128), ("delta", 16), ("delta", 32)])
+@pytest.mark.parametrize("bad", [np.inf, -np.inf, np.nan])
+def test_non_finite_activation_stays_in_its_row_and_columns(kind, split, bad):
+    """One Inf / NaN at X[0][k]: only the outputs C[0][n] of columns n that gather row k may be non-finite.
+    Rows 1.. (other sequences of the batch) and the columns that do not gather k equal the fp64 oracle to the
+    usual 1e-3 -- in particular on the four-row fp16 tiles, whose sums run on the matrix unit when all is finite."""
+    K, N, S = 2560, 640, 1536
+    _, pos, neg = matrix(K, N, S)
+    w = sp.Weights.upload_u16(pos, neg, K, split) if kind == "u16" else sp.Weights.upload_delta(pos, neg, K, split)
+    for M, dtype in ((4, np.float16), (3, np.float16), (1, np.float16), (4, np.float32)):
+        for k in (0, 1337, K - 1):
+            say("non-finite", kind, split, dtype.__name__, "M", M, "k", k, bad)
+            X = oracle.make_x_normal(500 + M + k, M, K, dtype)
+            X[0, k] = bad
+            clean = X.copy()
+            clean[0, k] = 0
+            ref = oracle.sptmm_f64(clean, pos, neg)
+            got = w.matmul(X)
+            away = finite_columns(pos, neg, k)
+            assert 0 < away.sum() < N
+            assert np.isfinite(got[1:]).all() and np.isfinite(got[0, away]).all()
+            check_fp(got[1:], ref[1:], S)
+            check_fp(got[0:1, away], ref[0:1, away], S)
+            assert (~np.isfinite(got[0, ~away])).all()  # Inf or NaN where the row is gathered, as IEEE sums give
+    w.free()
+
+
+def test_non_finite_activation_batched_launch_only_touches_its_own_gemv():
+    K, N, S = 2560, 640, 1536
+    _, pos, neg = matrix(K, N, S)
+    w = sp.Weights.upload_u16(pos, neg, K, 32)
+    Xs = [oracle.make_x_normal(900 + i, 4, K, np.float16) for i in range(3)]
+    Xs[1][2, 77] = np.inf
+    xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
+    cb = [sp.DeviceBuffer(4 * 4 * N) for _ in Xs]
+    say("non-finite batched")
+    sp.gemv_batched([w, w, w], xb, cb, 4, 1)
+    sp.device_sync()
+    for i in (0, 2):
+        check_fp(cb[i].to_numpy(np.float32, (4, N)), oracle.sptmm_f64(Xs[i], pos, neg), S)
+    got = cb[1].to_numpy(np.float32, (4, N))
+    clean = Xs[1].copy()
+    clean[2, 77] = 0
+    ref = oracle.sptmm_f64(clean, pos, neg)
+    away = finite_columns(pos, neg, 77)
+    check_fp(got[[0, 1, 3]], ref[[0, 1, 3]], S)
+    check_fp(got[2:3, away], ref[2:3, away], S)
+    assert (~np.isfinite(got[2, ~away])).all()
+    for o in [w] + xb + cb:
+        o.free()
+
+
 # ------------------------------------------------------------------------ i2s
 @pytest.mark.parametrize("K,N,S", [(6912, 2560, 4096), (2560, 2560, 1536), (2560, 640, 1536),
                                    (2560, 6912, 1536), (304, 32, 100), (512, 48, 256), (64, 16, 32)])
@@ -310,6 +369,43 @@ def test_decoder_layer_shapes_all_formats(name, K, N, S):
             assert (w.matmul(X) == want).all(), (name, w.info, M)
     for w in ws:
         w.free()
+
+
+# The fused projections the reference times (main.cu:1107-1120 for the lists at N = 13824, main.cu:1916-1917 for
+# i2s at N = 3840): q+k+v as one K=2560 -> N=3840 matrix, gate+up as one K=2560 -> N=13824 matrix.  N = 13824 at
+# split 32 is 6,912 tasks: several workgroups per compute unit and more than one task per wavefront in one launch.
+FUSED = [("q+k+v", 2560, 3840, 1536), ("gate+up", 2560, 13824, 1536)]
+
+
+@pytest.mark.parametrize("name,K,N,S", FUSED)
+def test_fused_projection_shapes_single_and_batched(name, K, N, S):
+    W, pos, neg = matrix(K, N, S, dense=True)
+    encodings = [("u16", s, lambda s=s: sp.Weights.upload_u16(pos, neg, K, s)) for s in (16, 32, 64)]
+    encodings += [("delta", s, lambda s=s: sp.Weights.upload_delta(pos, neg, K, s)) for s in (16, 32)]
+    encodings += [("i2s", 0, lambda: sp.Weights.upload_i2s(W))]
+    Xs = {M: [x_i8(7000 + 10 * M + i, M, K) for i in range(3)] for M in (1, 4, 8)}
+    want = {M: [oracle.sptmm_i8_mt(x, pos, neg, 8) for x in Xs[M]] for M in Xs}
+    st = sp.Stream()
+    for kind, split, make in encodings:
+        w = make()
+        ws = [w, w.clone(), w.clone()]
+        for M in (1, 4, 8):
+            say("fused", name, kind, "split", split, "M", M, "single")
+            assert (w.matmul(Xs[M][0]) == want[M][0]).all(), (kind, split, M)
+            say("fused", name, kind, "split", split, "M", M, "batched x3")
+            xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs[M]]
+            cb = [sp.DeviceBuffer(4 * M * N) for _ in ws]
+            for c in cb:
+                c.fill(0xFF)
+            sp.gemv_i8_batched(ws, xb, cb, M, st)
+            st.sync()
+            for i in range(3):
+                assert (cb[i].to_numpy(np.int32, (M, N)) == want[M][i]).all(), (kind, split, M, i)
+            for o in xb + cb:
+                o.free()
+        for o in ws:
+            o.free()
+    st.destroy()
 
 
 def test_large_layer_config4_three_encodings():
@@ -365,6 +461,24 @@ def test_tile_limit_and_largest_k():
                 with pytest.raises(sp.SptmmError) as e:
                     w.matmul(X)
                 assert e.value.code == -2 and "LDS" in str(e.value)
+            w.free()
+
+
+def test_eight_row_tiles_up_to_the_last_k_that_fits():
+    """Eight-row int8 tiles take 8 bytes of LDS per row of K plus what the workgroup keeps behind the tile; where
+    that no longer fits, the launch falls back to four-row tiles instead of failing (K around 20,400)."""
+    N, S = 32, 512
+    for K in (20352, 20368, 20384, 20400, 20416):
+        _, pos, neg = sp.generate_ternary(K, N, S)
+        X = x_i8(K, 8, K)
+        want = oracle.sptmm_i8(X, pos, neg)
+        for w in (sp.Weights.upload_u16(pos, neg, K, 32), sp.Weights.upload_u16(pos, neg, K, 256), sp.Weights.upload_delta(pos, neg, K, 32)):
+            say("eight-row limit K", K, w.info["kind"], w.info["split_k"])
+            assert (w.matmul(X) == want).all()
+            Xh = oracle.make_x_normal(K, 8, K, np.float32).astype(np.float16)
+            q, a = oracle.quantise_rows(Xh.astype(np.float32))
+            got = w.matmul_q8(Xh, w_scale=0.5)
+            assert (got == oracle.rescale(oracle.sptmm_i8(q, pos, neg), a, 0.5)).all()
             w.free()
 
 
