@@ -287,7 +287,7 @@ namespace {
 struct FileHeader {
     char magic[8];            // "SPTMMW1\0"
     uint32_t header_bytes;    // sizeof(FileHeader)
-    uint32_t version;         // 1
+    uint32_t version;         // 2 (1: i2s tiles in the older lane order, column-major inside a tile; re-tiled on load)
     int32_t kind, K, N, S, split_k, delta_bits, ragged;
     int32_t half, L, G, W, n_lane, tasks;
     int32_t task_stride, counts_bytes, n_min, n_max, index_shift;
@@ -319,7 +319,7 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
         FileHeader h{};
         memcpy(h.magic, FILE_MAGIC, 8);
         h.header_bytes = (uint32_t)sizeof h;
-        h.version = 1;
+        h.version = 2;
         const sptmm_winfo &i = w->info;
         const Geometry &g = w->geo;
         h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = i.ragged;
@@ -344,7 +344,7 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         FileHeader h{};
         std::vector<uint8_t> host;
         int rc = SPTMM_OK;
-        if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || h.version != 1)
+        if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || (h.version != 1 && h.version != 2))
             rc = fail(SPTMM_ERR_INVALID, "%s is not a weight file of this library", path);
         // every field the kernels index with is checked against the stream size before anything is uploaded
         if (!rc) {
@@ -389,6 +389,15 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         }
         fclose(f);
         if (rc) return rc;
+        if (h.version == 1 && h.kind == SPTMM_KIND_I2S) {
+            // version 1 kept the 16-byte unit of (column c, quarter q) at position 4c + q of its 1 KiB tile; now 16q + c
+            std::vector<uint8_t> tile(1024);
+            for (size_t t = 0; t + 1024 <= host.size(); t += 1024) {
+                memcpy(tile.data(), host.data() + t, 1024);
+                for (int c = 0; c < 16; ++c)
+                    for (int q = 0; q < 4; ++q) memcpy(host.data() + t + (size_t)(16 * q + c) * 16, tile.data() + (size_t)(4 * c + q) * 16, 16);
+            }
+        }
         if (h.ragged && (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA)) {
             // the per-task counts are what the kernel trusts most: keep them inside [n_min, n_max]
             const uint32_t *pre = (const uint32_t *)host.data();

@@ -662,11 +662,12 @@ size_t sptmm_pack_i2s_bytes(int K, int N)
 }
 
 // Word index of rows [16*g16, 16*g16+16) of column c: tiles of 16 columns x 256
-// rows (1 KiB); inside a tile lane = (c%16)*4 + quarter, 4 words per lane.
+// rows (1 KiB); inside a tile lane = quarter*16 + c%16, 4 words per lane -- the order in which
+// a 16x16x64 matrix instruction takes its B operand (column = lane mod 16, k-block = lane / 16).
 static inline size_t i2s_word_index(int Kp, int c, int g16)
 {
     int rounds = Kp / 256, r = g16 / 16, q = (g16 % 16) / 4, j = g16 % 4;
-    return ((size_t)(c / 16) * rounds + r) * 256 + (size_t)((c % 16) * 4 + q) * 4 + j;
+    return ((size_t)(c / 16) * rounds + r) * 256 + (size_t)(q * 16 + c % 16) * 4 + j;
 }
 
 int sptmm_pack_i2s(const int8_t *W, int K, int N, void *out)

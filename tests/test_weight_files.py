@@ -76,3 +76,38 @@ def test_save_load_round_trip_every_encoding(tmp_path):
         open(path, "wb").write(bytes(bad))
         with pytest.raises(sp.SptmmError):
             sp.Weights.load(path)
+
+
+def _fnv1a(data: bytes) -> int:
+    h = 1469598103934665603
+    for b in data:
+        h = ((h ^ b) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+@pytest.mark.gpu
+def test_version_1_i2s_file_is_retiled_on_load(tmp_path):
+    """Files of format version 1 kept the 16-byte unit of (column c, quarter q) at position 4c + q of its 1 KiB
+    tile; the stream now keeps it at 16q + c.  A version-1 file is rebuilt here from a fresh one and must load
+    to the same matrix."""
+    sp.device_init(0)
+    K, N, S = 512, 48, 256
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    X = oracle.make_x_i8(3, 5, K)
+    w = sp.Weights.upload_i2s(W)
+    path = str(tmp_path / "new.sptmm")
+    w.save(path)
+    w.free()
+    raw = bytearray(open(path, "rb").read())
+    assert int.from_bytes(raw[12:16], "little") == 2
+    stream = np.frombuffer(bytes(raw[120:]), np.uint8).reshape(-1, 4, 16, 16)      # [tile][q][c][16 bytes]
+    old = np.ascontiguousarray(stream.transpose(0, 2, 1, 3)).tobytes()             # [tile][c][q][16 bytes]
+    hdr = bytearray(raw[:120])
+    hdr[12:16] = (1).to_bytes(4, "little")
+    hdr[112:120] = bytes(8)
+    hdr[112:120] = _fnv1a(bytes(hdr) + old).to_bytes(8, "little")
+    p1 = str(tmp_path / "v1.sptmm")
+    open(p1, "wb").write(bytes(hdr) + old)
+    v = sp.Weights.load(p1)
+    assert (v.matmul(X) == oracle.dense_i8(X, W)).all()
+    v.free()
