@@ -284,7 +284,21 @@ def main():
                 sums.append(tot)
         configs["cfg3_layer"] = {"shapes": rows, "summed_layer": sums}
     if "cfg4" in legs:
-        configs["cfg4_large"] = run_matrix(*LARGE, (1, 8, 16))
+        rows = run_matrix(*LARGE, (1, 8, 16))
+        # the same matrix as wide streams (K-tiled, 16-row tiles): the lists read once at M = 16, where the ordinary
+        # streams take two passes of eight rows because a 16-row tile of K = 13824 does not fit the LDS
+        name, k_rows, n_cols, s_nz = LARGE
+        Wl = sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)[0]
+        X16 = sp.make_x_i8(0xC0FFEE ^ 16, 16, k_rows)
+        ref16 = next(g for lab, xx, _, _, g, _ in checks if lab == "large M=16")
+        for enc, kind in (("wide u16/32", sp.KIND_U16), ("wide delta/32", sp.KIND_DELTA)):
+            ww = sp.Weights.upload_wide(Wl, kind, 32)
+            r = {"shape": name, "K": k_rows, "N": n_cols, "S": s_nz, "M": 16, "enc": enc, "k_tile": ww.info["k_tile"],
+                 "bit_exact_across_encodings": bool((ww.matmul(X16) == ref16).all())}
+            r.update(time_encoding(ww, 0, X16, 16, n_cols, k_rows))
+            rows.append(r)
+            ww.free()
+        configs["cfg4_large"] = rows
 
     gbps = nbytes / us_gemv / 1e3
     traffic, traffic_src = None, None

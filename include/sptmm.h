@@ -59,6 +59,7 @@ typedef struct sptmm_winfo {
     uint64_t stream_bytes; /* bytes of the weight stream one GEMV reads */
     int ragged;      /* 1: built from a matrix whose columns differ in nonzeros (S is 0 then) */
     uint64_t nnz;    /* nonzeros of the whole matrix */
+    int k_tile;      /* wide streams: rows per K-tile (0 for every other stream) */
 } sptmm_winfo;
 
 typedef struct sptmm_weights sptmm_weights; /* opaque; owns its device buffer */
@@ -126,6 +127,19 @@ int sptmm_generate_ternary_iid(int K, int N, uint32_t seed, double p_pos, double
  * at words[n*(K/16) + g] holds rows 16g..16g+15 (main.cu:176-196). */
 int sptmm_dense_from_i2s_words(const uint32_t *words, int K, int N, int8_t *W_colmajor);
 
+/* Wide streams: u16 lists or gap streams for activation tiles of 16 int8 rows (8 fp16 rows), cut
+ * into K-tiles of k_tile rows so that such a tile fits the LDS: the stream is read ONCE for up to
+ * 16 rows whatever K is (the reference reads its lists once per row, main.cu:567, and this
+ * library's other streams once per 8 rows when a 16-row tile does not fit).  Any K x N matrix over
+ * {-1,0,+1}; split_k in {8,16,32,64}; k_tile a multiple of 16 (sptmm_wide_k_tile gives the largest
+ * that fits an LDS of the given size).  *bits as in the ragged packer.  The stream is
+ * self-describing (a 512-byte header with the K-tile table; at most 16 K-tiles). */
+int sptmm_wide_k_tile(int K, int lds_bytes);
+size_t sptmm_pack_wide_bytes(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int k_tile, int *bits, size_t *read_bytes,
+                             uint64_t *nnz);
+int sptmm_pack_wide(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int k_tile, int bits, void *out);
+int sptmm_unpack_wide(const void *packed, int K, int N, int8_t *W_colmajor);
+
 /* i2s: 16 weights per word, code = w + 2, element e at bit 8*(e%4) + 2*(e/4)
  * (main.cu:176-192, decode bitnet_kernels.cuh:52-72).  Word order is this
  * library's own wave64 tiling, not the reference's (whose prepared matrix,
@@ -150,6 +164,10 @@ int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weigh
  * ragged gap stream, or i2s).  The GEMV entry points below serve it like any
  * other weights object. */
 int sptmm_weights_upload_dense(const int8_t *W_colmajor, int K, int N, int kind, int split_k, sptmm_weights **out);
+/* Any ternary matrix -> wide device stream (u16 lists or gap stream), K-tiled for this device's
+ * LDS.  sptmm_gemv_i8 and sptmm_gemv_f16 (and the batched call) serve it with 16-row (8-row) tiles:
+ * meant for M > 8 (M > 4 with fp16 rows); correct for any M.  No counterpart in the reference. */
+int sptmm_weights_upload_wide(const int8_t *W_colmajor, int K, int N, int kind, int split_k, sptmm_weights **out);
 /* Second device copy of the same stream (used to rotate over more bytes than
  * the last-level cache holds when timing cold reads).  The copy is complete on
  * return: a launch on any stream may follow at once. */

@@ -9,7 +9,7 @@ import numpy as np
 __all__ = [
     "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
-    "generate_ternary_iid", "dense_from_i2s_words",
+    "generate_ternary_iid", "dense_from_i2s_words", "wide_k_tile", "pack_wide", "unpack_wide",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
     "device_sync", "Graph", "measure_gemv", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
@@ -25,6 +25,7 @@ EXPORTS = [
     "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
     "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_pack_ragged_bytes", "sptmm_pack_ragged",
     "sptmm_unpack_ragged", "sptmm_generate_ternary_iid", "sptmm_dense_from_i2s_words", "sptmm_weights_upload_dense",
+    "sptmm_wide_k_tile", "sptmm_pack_wide_bytes", "sptmm_pack_wide", "sptmm_unpack_wide", "sptmm_weights_upload_wide",
     "sptmm_device_init",
     "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
@@ -52,7 +53,7 @@ class DevInfo(C.Structure):
 class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
                 ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64),
-                ("ragged", C.c_int), ("nnz", C.c_uint64)]
+                ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int)]
 
 
 def lib_path() -> str:
@@ -71,7 +72,7 @@ def lib() -> C.CDLL:
         L.sptmm_last_error.restype = C.c_char_p
         L.sptmm_version.restype = C.c_char_p
         for n in ("sptmm_pack_u16_bytes", "sptmm_pack_delta_bytes", "sptmm_pack_i2s_bytes", "sptmm_weights_bytes",
-                  "sptmm_pack_ragged_bytes"):
+                  "sptmm_pack_ragged_bytes", "sptmm_pack_wide_bytes"):
             getattr(L, n).restype = C.c_size_t
         L.sptmm_i2s_pack_word.restype = C.c_uint32
         L.sptmm_i2s_decode_word.restype = None
@@ -251,6 +252,28 @@ def pack_ragged(W: np.ndarray, kind: int, split_k: int, bits: int = 0):
 def unpack_ragged(packed: np.ndarray, K: int, N: int, kind: int, split_k: int, bits: int = 0) -> np.ndarray:
     W = np.empty((N, K), np.int8)
     _ck(lib().sptmm_unpack_ragged(_p(packed), K, N, kind, split_k, bits, _p(W)))
+    return W
+
+
+def wide_k_tile(K: int, lds_bytes: int = 160 * 1024) -> int:
+    return _ck(lib().sptmm_wide_k_tile(K, lds_bytes))
+
+
+def pack_wide(W: np.ndarray, kind: int, split_k: int, k_tile: int, bits: int = 0):
+    """Any ternary matrix W [N][K] -> (wide stream bytes, dict(bits, read_bytes, nnz))."""
+    N, K = W.shape
+    b, rb, nnz = C.c_int(bits), C.c_size_t(), C.c_uint64()
+    n = lib().sptmm_pack_wide_bytes(_p(W), K, N, kind, split_k, k_tile, C.byref(b), C.byref(rb), C.byref(nnz))
+    if not n:
+        raise SptmmError(-1, lib().sptmm_last_error().decode())
+    out = np.zeros(n, np.uint8)
+    _ck(lib().sptmm_pack_wide(_p(W), K, N, kind, split_k, k_tile, b.value, _p(out)))
+    return out, {"bits": b.value, "read_bytes": rb.value, "nnz": nnz.value}
+
+
+def unpack_wide(packed: np.ndarray, K: int, N: int) -> np.ndarray:
+    W = np.empty((N, K), np.int8)
+    _ck(lib().sptmm_unpack_wide(_p(packed), K, N, _p(W)))
     return W
 
 
@@ -453,6 +476,14 @@ class Weights:
         N, K = W.shape
         h = C.c_void_p()
         _ck(lib().sptmm_weights_upload_dense(_p(W), K, N, kind, split_k, C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def upload_wide(cls, W: np.ndarray, kind: int, split_k: int = 32) -> "Weights":
+        """Any ternary matrix W [N][K] as a wide stream (K-tiled, 16 int8 / 8 fp16 rows per tile): for M > 8."""
+        N, K = W.shape
+        h = C.c_void_p()
+        _ck(lib().sptmm_weights_upload_wide(_p(W), K, N, kind, split_k, C.byref(h)))
         return cls(h)
 
     def save(self, path: str):

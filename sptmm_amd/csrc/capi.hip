@@ -23,6 +23,8 @@ struct sptmm_weights {
     int task_stride = 0, counts_bytes = 0;  // ragged streams
     int n_min = 0, n_max = 0;
     int index_shift = 0;  // u16 streams: fields are row << index_shift
+    bool wide = false;    // wide stream (K-tiled, 16-byte slots): `wh` describes it
+    WideHeader wh;
 };
 
 namespace {
@@ -124,6 +126,10 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.batch_w = bw;
     a.batch_X = bx;
     a.batch_C = bc;
+    if (w->wide) {
+        if (quant) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
+        return launch_wide(a, w->wh, act, stream);
+    }
     switch (w->info.kind) {
     case SPTMM_KIND_U16: return launch_u16(a, act, stream);
     case SPTMM_KIND_DELTA: return launch_delta(a, act, stream);
@@ -244,6 +250,37 @@ int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int spli
     });
 }
 
+int sptmm_weights_upload_wide(const int8_t *W, int K, int N, int kind, int split_k, sptmm_weights **out)
+{
+    return guarded([&]() -> int {
+        if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        DevCaps caps;
+        if (int rc = device_caps(&caps)) return rc;
+        const int k_tile = sptmm_wide_k_tile(K, caps.lds);
+        if (k_tile < 0) return k_tile;
+        int bits = 0;
+        size_t read_bytes = 0;
+        uint64_t nnz = 0;
+        const size_t bytes = sptmm_pack_wide_bytes(W, K, N, kind, split_k, k_tile, &bits, &read_bytes, &nnz);
+        if (!bytes) return SPTMM_ERR_INVALID;  // message set by the planner
+        std::vector<uint8_t> host(bytes);
+        if (int rc = sptmm_pack_wide(W, K, N, kind, split_k, k_tile, bits, host.data())) return rc;
+        sptmm_weights *w = new (std::nothrow) sptmm_weights();
+        if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
+        w->info = sptmm_winfo{kind, K, N, 0, split_k, bits, read_bytes, 1, nnz, k_tile};
+        w->wide = true;
+        if (int rc = wide_parse_header(host.data(), &w->wh)) {
+            delete w;
+            return rc;
+        }
+        if (int rc = make_ragged_geometry(N, split_k, 64, &w->geo)) {
+            delete w;
+            return rc;
+        }
+        return finish_upload(w, host, out);
+    });
+}
+
 int sptmm_weights_clone(const sptmm_weights *w, sptmm_weights **out)
 {
     return guarded([&]() -> int {
@@ -314,6 +351,7 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
 {
     return guarded([&]() -> int {
         if (!w || !path) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (w->wide) return fail(SPTMM_ERR_UNSUPPORTED, "wide streams are tied to the LDS size of the device they were packed for and are not saved");
         std::vector<uint8_t> host(w->bytes);
         HIP_TRY(hipMemcpy(host.data(), w->dev, w->bytes, hipMemcpyDeviceToHost));
         FileHeader h{};
@@ -437,7 +475,8 @@ int sptmm_gemv_batched(const sptmm_weights *const *ws, const void *const *X, voi
             if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
             const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
             if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
-                a.ragged != b.ragged || ws[0]->task_stride != ws[i]->task_stride ||
+                a.ragged != b.ragged || a.k_tile != b.k_tile || ws[0]->wide != ws[i]->wide ||
+                (ws[0]->wide && memcmp(&ws[0]->wh, &ws[i]->wh, sizeof(WideHeader)) != 0) || ws[0]->task_stride != ws[i]->task_stride ||
                 ws[0]->n_min != ws[i]->n_min)
                 return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);
             wp[i] = ws[i]->dev;

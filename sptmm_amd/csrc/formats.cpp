@@ -215,11 +215,11 @@ namespace sptmm {
 
 void schedule(Domain &d)
 {
-    const int no = d.owners, Lo = d.lanes, n = d.n;
+    const int no = d.owners, Lo = d.lanes, n = d.n, NB = d.banks, mask = d.banks - 1;
     std::vector<std::array<std::vector<uint16_t>, 32>> pool(no);
     std::vector<int> wild(no);  // padding cells of each owner, free to take any bank
     for (int o = 0; o < no; ++o) {
-        for (uint16_t k : d.entries[o]) pool[o][k & 31].push_back(k);
+        for (uint16_t k : d.entries[o]) pool[o][k & mask].push_back(k);
         wild[o] = n * Lo - (int)d.entries[o].size();
     }
     d.cell.assign(no, std::vector<uint16_t>((size_t)n * Lo));
@@ -234,13 +234,13 @@ void schedule(Domain &d)
         }
         while (open > 0) {  // one sweep = one more entry allowed per bank
             int order[32], total[32];
-            for (int b = 0; b < 32; ++b) {
+            for (int b = 0; b < NB; ++b) {
                 order[b] = b;
                 total[b] = 0;
                 for (int o = 0; o < no; ++o) total[b] += (int)pool[o][b].size();
             }
-            std::sort(order, order + 32, [&](int x, int y) { return total[x] != total[y] ? total[x] > total[y] : x < y; });
-            for (int i = 0; i < 32 && open > 0; ++i) {
+            std::sort(order, order + NB, [&](int x, int y) { return total[x] != total[y] ? total[x] > total[y] : x < y; });
+            for (int i = 0; i < NB && open > 0; ++i) {
                 const int b = order[i];
                 int who = -1;
                 for (int o = 0; o < no; ++o)
@@ -249,7 +249,7 @@ void schedule(Domain &d)
                     for (int o = 0; o < no; ++o)
                         if (need[o] > 0 && wild[o] > 0 && (who < 0 || wild[o] > wild[who])) who = o;
                     if (who < 0) continue;
-                    pick[who].push_back((uint16_t)(d.zero_base + ((b - d.zero_base) & 31)));
+                    pick[who].push_back((uint16_t)(d.zero_base + ((b - d.zero_base) & mask)));
                     --wild[who];
                 } else {
                     pick[who].push_back(pool[who][b].back());
@@ -260,7 +260,7 @@ void schedule(Domain &d)
             }
         }
         for (int o = 0; o < no; ++o) {
-            std::sort(pick[o].begin(), pick[o].end(), [](uint16_t x, uint16_t y) { return (x & 31) != (y & 31) ? (x & 31) < (y & 31) : x < y; });
+            std::sort(pick[o].begin(), pick[o].end(), [mask](uint16_t x, uint16_t y) { return (x & mask) != (y & mask) ? (x & mask) < (y & mask) : x < y; });
             for (int l = 0; l < Lo; ++l) d.cell[o][(size_t)slot * Lo + l] = pick[o][l];
         }
     }
@@ -268,7 +268,7 @@ void schedule(Domain &d)
 
 bool schedule_runs(RunDomain &d, int window)
 {
-    const int n = d.n;
+    const int n = d.n, NL = d.lanes, mask = d.lanes - 1;  // lanes of the domain = banks it spreads over
     struct Lane {
         std::vector<char> seen;   // visited entries
         int lo = 0, cur = -1;     // oldest entry not visited yet; row visited last
@@ -276,12 +276,12 @@ bool schedule_runs(RunDomain &d, int window)
         int pick = -1;
     } lane[32];
     int demand[32] = {0};         // rows still to visit, per bank, over the whole domain
-    for (int l = 0; l < 32; ++l) {
+    for (int l = 0; l < NL; ++l) {
         if ((int)d.rows[l].size() != n) return false;
         for (int i = 1; i < n; ++i)
             if (d.rows[l][i] - d.rows[l][i - 1] > 127) return false;
         for (int i = 0; i < n; ++i)
-            if (d.rows[l][i] < d.zero_row) ++demand[d.rows[l][i] & 31];
+            if (d.rows[l][i] < d.zero_row) ++demand[d.rows[l][i] & mask];
         lane[l].seen.assign(n, 0);
         d.order[l].assign(n, 0);
     }
@@ -290,7 +290,7 @@ bool schedule_runs(RunDomain &d, int window)
     struct Matcher {
         Lane *lane;
         RunDomain &d;
-        int cap = 1;
+        int cap = 1, mask = 31;
         int owners[32][32], count[32];
         bool tried[32];
         bool place(int l)
@@ -301,7 +301,7 @@ bool schedule_runs(RunDomain &d, int window)
                     lane[l].pick = i;
                     return true;
                 }
-                const int b = row & 31;
+                const int b = row & mask;
                 if (tried[b]) continue;
                 tried[b] = true;
                 if (count[b] < cap) {
@@ -319,17 +319,18 @@ bool schedule_runs(RunDomain &d, int window)
             return false;
         }
     } m{lane, d};
+    m.mask = mask;
 
     double credit = 0.0;
     for (int step = 0; step < n; ++step) {
         // A bank asked for more often than there are steps left has to be served more than once
         // per step at some point; doing that at an even rate costs the fewest passes overall.
         double q = 1.0;
-        for (int b = 0; b < 32; ++b) q = std::max(q, (double)demand[b] / (n - step));
+        for (int b = 0; b < NL; ++b) q = std::max(q, (double)demand[b] / (n - step));
         credit += q;
         const int cap = std::max(1, (int)credit);  // e.g. q = 1.3: one step in three serves every bank twice
         credit -= cap;
-        for (int l = 0; l < 32; ++l) {
+        for (int l = 0; l < NL; ++l) {
             Lane &L = lane[l];
             const std::vector<uint16_t> &r = d.rows[l];
             L.cand.clear();
@@ -351,31 +352,31 @@ bool schedule_runs(RunDomain &d, int window)
             }
             if (L.cand.empty()) return false;  // cannot happen while the sorted gaps fit; kept as a guard
             std::stable_sort(L.cand.begin(), L.cand.end(), [&](int x, int y) {
-                const int dx = r[x] >= d.zero_row ? -1 : demand[r[x] & 31], dy = r[y] >= d.zero_row ? -1 : demand[r[y] & 31];
+                const int dx = r[x] >= d.zero_row ? -1 : demand[r[x] & mask], dy = r[y] >= d.zero_row ? -1 : demand[r[y] & mask];
                 return dx > dy;
             });
         }
         m.cap = cap;
-        for (int b = 0; b < 32; ++b) m.count[b] = 0;
+        for (int b = 0; b < NL; ++b) m.count[b] = 0;
         int load[32] = {0};
         bool placed[32];
-        for (int l = 0; l < 32; ++l) {
-            for (int b = 0; b < 32; ++b) m.tried[b] = false;
+        for (int l = 0; l < NL; ++l) {
+            for (int b = 0; b < NL; ++b) m.tried[b] = false;
             placed[l] = m.place(l);
         }
-        for (int b = 0; b < 32; ++b) load[b] = m.count[b];
-        for (int l = 0; l < 32; ++l) {
+        for (int b = 0; b < NL; ++b) load[b] = m.count[b];
+        for (int l = 0; l < NL; ++l) {
             Lane &L = lane[l];
             if (!placed[l]) {  // no bank with room: join the least loaded one
                 int best = L.cand[0];
                 for (int i : L.cand)
-                    if (load[d.rows[l][i] & 31] < load[d.rows[l][best] & 31]) best = i;
+                    if (load[d.rows[l][i] & mask] < load[d.rows[l][best] & mask]) best = i;
                 L.pick = best;
-                ++load[d.rows[l][best] & 31];
+                ++load[d.rows[l][best] & mask];
             }
             L.seen[L.pick] = 1;
             L.cur = d.rows[l][L.pick];
-            if (L.cur < d.zero_row) --demand[L.cur & 31];
+            if (L.cur < d.zero_row) --demand[L.cur & mask];
             d.order[l][step] = (uint16_t)L.cur;
             while (L.lo < n && L.seen[L.lo]) ++L.lo;
         }

@@ -87,6 +87,7 @@ int u16_index_shift(int K);
 // behind the activation tile.
 struct Domain {
     int owners = 0, lanes = 0, n = 0;
+    int banks = 32;  // owners * lanes; 16 for the 16-byte slots of the wide tiles (the LDS serves 16 lanes of a b128 read per pass)
     int zero_base = 0;
     std::vector<std::vector<uint16_t>> entries;  // per owner
     std::vector<std::vector<uint16_t>> cell;     // per owner: [slot][lane] -> row
@@ -104,6 +105,7 @@ void schedule(Domain &d);
 // 8-bit stream exists then).
 struct RunDomain {
     int n = 0, zero_row = 0;
+    int lanes = 32;  // lanes scheduled together = banks (row mod lanes) they are spread over; 16 for the wide tiles
     std::vector<uint16_t> rows[32];
     std::vector<uint16_t> order[32];
 };
@@ -121,6 +123,14 @@ int ragged_index_shift(int K);
 // count per task; the tasks follow at the next multiple of 256 bytes
 constexpr uint32_t RAGGED_MAGIC = 0x52545053u;  // "SPTR"
 inline size_t ragged_counts_bytes(int tasks) { return ((size_t)16 + 2 * (size_t)tasks + 255) / 256 * 256; }
+
+// Wide streams (wide.cpp): what the 512-byte header in front of the K-tiles' sub-streams says.
+struct WideHeader {
+    int phases = 0, k_tile = 0, K = 0, N = 0, kind = 0, bits = 0, split_k = 0;
+    uint32_t offset[16] = {0}, stride[16] = {0};
+    int n_min[16] = {0}, n_max[16] = {0};
+};
+int wide_parse_header(const void *packed, WideHeader *out);
 
 // i2s tiling: 16 columns x 4 lanes per wave-load, 16 bytes (64 weights) per lane.
 inline int i2s_padded_k(int K) { return (K + 255) / 256 * 256; }
@@ -162,6 +172,7 @@ int launch_ragged_u16_plain(const GemvArgs &a, ActType act, void *stream);   // 
 int launch_ragged_runs8(const GemvArgs &a, ActType act, void *stream);       // lists_ragged_runs8.hip
 int launch_ragged_runs16(const GemvArgs &a, ActType act, void *stream);      // lists_ragged_runs16.hip
 int launch_delta(const GemvArgs &a, ActType act, void *stream);
+int launch_wide(const GemvArgs &a, const WideHeader &h, ActType act, void *stream);  // lists_wide.hip
 int launch_i2s(const GemvArgs &a, void *stream);
 int launch_copy(void *dst, const void *src, size_t bytes, void *stream);
 int launch_read(const void *src, size_t bytes, void *sink, int workgroups, void *stream);
