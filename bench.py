@@ -160,12 +160,13 @@ def main():
                 "batched_us": round(bat, 3), "batched_gbps": round(nb / bat / 1e3, 1), "batched_pct_roofline": pct(nb, bat),
                 "gemvs_per_batched_launch": len(groups[0])}
 
-    def run_matrix(label, k_rows, n_cols, s_nz, ms, lists=None):
-        """The three encodings of one seeded matrix at the given row counts -> list of rows."""
+    def run_matrix(label, k_rows, n_cols, s_nz, ms, lists=None, split=0):
+        """The three encodings of one seeded matrix at the given row counts -> list of rows.  split = 0: the split
+        the library picks for the shape (sptmm_choose_split_k); the row's `split_k` says which."""
         Wm, p, n = lists if lists is not None else sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)
         rows = []
-        makers = (("u16/32", lambda: sp.Weights.upload_u16(p, n, k_rows, 32)),
-                  ("delta/32", lambda: sp.Weights.upload_delta(p, n, k_rows, 32)),
+        makers = (("u16", lambda: sp.Weights.upload_u16(p, n, k_rows, split)),
+                  ("delta", lambda: sp.Weights.upload_delta(p, n, k_rows, split)),
                   ("i2s", lambda: sp.Weights.upload_i2s(Wm)))
         refs = {}
         for enc, mk in makers:
@@ -176,7 +177,7 @@ def main():
                 if m not in refs:
                     refs[m] = got
                     checks.append(("%s M=%d" % (label, m), Xm, p, n, got, s_nz))
-                r = {"shape": label, "K": k_rows, "N": n_cols, "S": s_nz, "M": m, "enc": enc,
+                r = {"shape": label, "K": k_rows, "N": n_cols, "S": s_nz, "M": m, "enc": enc, "split_k": w.info["split_k"],
                      "bit_exact_across_encodings": bool((got == refs[m]).all())}
                 r.update(time_encoding(w, 0, Xm, m, n_cols, k_rows))
                 rows.append(r)
@@ -254,7 +255,7 @@ def main():
     configs = {}
     if "cfg1" in legs:
         # config 1: the same matrix at four activation rows (indices still read once per GEMV)
-        configs["cfg1_m4"] = run_matrix("headline", K, N, S, (4,), (Wd, pos, neg))
+        configs["cfg1_m4"] = run_matrix("headline", K, N, S, (4,), (Wd, pos, neg), SPLIT)
     if "cfg2" in legs:
         # config 2: gap stream, fp16 rows ~N(0,1), fp32 sums
         rng = np.random.default_rng(2)
@@ -264,7 +265,7 @@ def main():
             Xh = rng.standard_normal((m, K)).astype(np.float16)
             got = ww.matmul(Xh)
             checks.append(("cfg2 fp16 M=%d" % m, Xh, pos, neg, got, S))
-            r = {"shape": "headline", "K": K, "N": N, "S": S, "M": m, "enc": "delta/32", "act": "fp16", "delta_bits": ww.info["delta_bits"]}
+            r = {"shape": "headline", "K": K, "N": N, "S": S, "M": m, "enc": "delta", "split_k": SPLIT, "act": "fp16", "delta_bits": ww.info["delta_bits"]}
             r.update(time_encoding(ww, 1, Xh, m, N, K))
             rows.append(r)
         ww.free()
@@ -275,7 +276,7 @@ def main():
             rows += run_matrix(name, k_rows, n_cols, s_nz, (1, 4), (Wd, pos, neg) if (k_rows, n_cols, s_nz) == (K, N, S) else None)
         sums = []
         for m in (1, 4):
-            for enc in ("u16/32", "delta/32", "i2s"):
+            for enc in ("u16", "delta", "i2s"):
                 tot = {"M": m, "enc": enc, "gemvs": sum(mult for *_, mult in LAYER)}
                 for key in ("alone_warm_us", "alone_cold_us", "batched_us", "bytes"):
                     tot[key] = round(sum(mult * next(r[key] for r in rows if (r["shape"], r["M"], r["enc"]) == (name, m, enc))
@@ -291,9 +292,9 @@ def main():
         Wl = sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)[0]
         X16 = sp.make_x_i8(0xC0FFEE ^ 16, 16, k_rows)
         ref16 = next(g for lab, xx, _, _, g, _ in checks if lab == "large M=16")
-        for enc, kind in (("wide u16/32", sp.KIND_U16), ("wide delta/32", sp.KIND_DELTA)):
+        for enc, kind in (("wide u16", sp.KIND_U16), ("wide delta", sp.KIND_DELTA)):
             ww = sp.Weights.upload_wide(Wl, kind, 32)
-            r = {"shape": name, "K": k_rows, "N": n_cols, "S": s_nz, "M": 16, "enc": enc, "k_tile": ww.info["k_tile"],
+            r = {"shape": name, "K": k_rows, "N": n_cols, "S": s_nz, "M": 16, "enc": enc, "split_k": 32, "k_tile": ww.info["k_tile"],
                  "bit_exact_across_encodings": bool((ww.matmul(X16) == ref16).all())}
             r.update(time_encoding(ww, 0, X16, 16, n_cols, k_rows))
             rows.append(r)

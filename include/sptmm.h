@@ -84,6 +84,13 @@ int sptmm_lists_from_dense(const int8_t *W_colmajor, int K, int N, int S, uint16
  * main.cu:784-797, which is unseeded): xorshift32 stream, r % 255 - 127. */
 int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X);
 
+/* The split_k this library would pick for a balanced matrix (kind: SPTMM_KIND_U16 or
+ * SPTMM_KIND_DELTA) on a device with `compute_units` CUs (0: 256) -- what the upload calls use when
+ * they are handed split_k = 0.  The reference leaves the choice to the command line
+ * (main.cu:998, 1042, 1059); the result does not depend on it.  Negative status when no split
+ * in 8..256 (gap streams: 8..64) divides S/2. */
+int sptmm_choose_split_k(int kind, int N, int S, int compute_units);
+
 /* Wave64 stream of the u16 lists; replaces the W_map_{8,16,32}_div layouts of
  * main.cu:343-374.  split_k in {8,16,32,64,128,256}; (S/2) % split_k == 0
  * (main.cu:564). */
@@ -156,7 +163,9 @@ int sptmm_unpack_i2s(const void *packed, int K, int N, int8_t *W_colmajor);
 int sptmm_device_init(int device, sptmm_devinfo *out);
 
 /* Host lists / dense matrix -> device stream.  Stand in for the cudaMalloc +
- * prepareW_map / prepareW_i2s sequence of main.cu:914-989 and 1851-1859. */
+ * prepareW_map / prepareW_i2s sequence of main.cu:914-989 and 1851-1859.
+ * split_k = 0 (here, in _upload_dense and in _upload_wide): sptmm_choose_split_k for the
+ * current device (ragged matrices: from the mean nonzeros per column). */
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weights **out);

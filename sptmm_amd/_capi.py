@@ -9,7 +9,7 @@ import numpy as np
 __all__ = [
     "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
-    "generate_ternary_iid", "dense_from_i2s_words", "wide_k_tile", "pack_wide", "unpack_wide",
+    "generate_ternary_iid", "dense_from_i2s_words", "choose_split_k", "wide_k_tile", "pack_wide", "unpack_wide",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
     "device_sync", "Graph", "measure_gemv", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
@@ -25,7 +25,7 @@ EXPORTS = [
     "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
     "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_pack_ragged_bytes", "sptmm_pack_ragged",
     "sptmm_unpack_ragged", "sptmm_generate_ternary_iid", "sptmm_dense_from_i2s_words", "sptmm_weights_upload_dense",
-    "sptmm_wide_k_tile", "sptmm_pack_wide_bytes", "sptmm_pack_wide", "sptmm_unpack_wide", "sptmm_weights_upload_wide",
+    "sptmm_choose_split_k", "sptmm_wide_k_tile", "sptmm_pack_wide_bytes", "sptmm_pack_wide", "sptmm_unpack_wide", "sptmm_weights_upload_wide",
     "sptmm_device_init",
     "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
@@ -253,6 +253,11 @@ def unpack_ragged(packed: np.ndarray, K: int, N: int, kind: int, split_k: int, b
     W = np.empty((N, K), np.int8)
     _ck(lib().sptmm_unpack_ragged(_p(packed), K, N, kind, split_k, bits, _p(W)))
     return W
+
+
+def choose_split_k(kind: int, N: int, S: int, compute_units: int = 0) -> int:
+    """The split_k the upload calls pick when handed 0."""
+    return _ck(lib().sptmm_choose_split_k(kind, N, S, compute_units))
 
 
 def wide_k_tile(K: int, lds_bytes: int = 160 * 1024) -> int:

@@ -61,6 +61,29 @@ int device_caps(DevCaps *c)
     return SPTMM_OK;
 }
 
+// split_k = 0 in an upload call: the library's own choice for this device
+int resolve_split(int kind, int N, int S, int *split_k)
+{
+    if (*split_k != 0) return SPTMM_OK;
+    DevCaps caps;
+    if (int rc = device_caps(&caps)) return rc;
+    const int s = sptmm_choose_split_k(kind, N, S, caps.cus);
+    if (s < 0) return s;
+    *split_k = s;
+    return SPTMM_OK;
+}
+// the same for an arbitrary ternary matrix: S = twice the mean nonzeros per column and sign, rounded to a multiple of 512
+int resolve_split_dense(const int8_t *W, int K, int N, int kind, int *split_k)
+{
+    if (*split_k != 0 || kind == SPTMM_KIND_I2S) return SPTMM_OK;
+    if (!W || K <= 0 || N <= 0) return fail(SPTMM_ERR_INVALID, "bad matrix");
+    size_t nnz = 0;
+    for (size_t i = 0, n = (size_t)K * N; i < n; ++i) nnz += W[i] != 0;
+    long S = (long)((nnz / (size_t)N + 511) / 512 * 512);
+    if (S < 512) S = 512;
+    return resolve_split(kind, (N + 15) / 16 * 16, (int)S, split_k);
+}
+
 int finish_upload(sptmm_weights *w, const std::vector<uint8_t> &host, sptmm_weights **out)
 {
     DevCaps caps;
@@ -174,6 +197,7 @@ int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, in
     return guarded([&]() -> int {
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
         if (int rc = check_shape(K, N, S)) return rc;
+        if (int rc = resolve_split(SPTMM_KIND_U16, N, S, &split_k)) return rc;
         Geometry g;
         if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
         std::vector<uint8_t> host(sptmm_pack_u16_bytes(N, S, split_k));
@@ -192,6 +216,7 @@ int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, 
     return guarded([&]() -> int {
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
         if (int rc = check_shape(K, N, S)) return rc;
+        if (int rc = resolve_split(SPTMM_KIND_DELTA, N, S, &split_k)) return rc;
         Geometry g;
         if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
         int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
@@ -227,6 +252,7 @@ int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int spli
     return guarded([&]() -> int {
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
         if (kind == SPTMM_KIND_I2S) return sptmm_weights_upload_i2s(W, K, N, out);
+        if (int rc = resolve_split_dense(W, K, N, kind, &split_k)) return rc;
         int bits = 0, n_min = 0, n_max = 0;
         size_t read_bytes = 0;
         uint64_t nnz = 0;
@@ -258,6 +284,8 @@ int sptmm_weights_upload_wide(const int8_t *W, int K, int N, int kind, int split
         if (int rc = device_caps(&caps)) return rc;
         const int k_tile = sptmm_wide_k_tile(K, caps.lds);
         if (k_tile < 0) return k_tile;
+        if (int rc = resolve_split_dense(W, K, N, kind, &split_k)) return rc;
+        if (split_k > 64) split_k = 64;
         int bits = 0;
         size_t read_bytes = 0;
         uint64_t nnz = 0;

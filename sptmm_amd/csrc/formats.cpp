@@ -409,6 +409,27 @@ void for_cells(const Geometry &g, int c, F f)
 
 extern "C" {
 
+int sptmm_choose_split_k(int kind, int N, int S, int compute_units)
+{
+    // Measured on MI355X over the decoder-layer shapes, K = 2560 ... 13824, N = 128 ... 13824: a lane does best with
+    // some 30 to 70 entries per sign (fewer and the per-task overhead shows, more and too few tasks are in flight),
+    // and a launch wants at least two tasks per compute unit -- small N pays for that with shorter lanes, down to 8.
+    const int max_split = kind == SPTMM_KIND_U16 ? 256 : 64;
+    if ((kind != SPTMM_KIND_U16 && kind != SPTMM_KIND_DELTA) || N <= 0 || S <= 0 || S % 2) return fail(SPTMM_ERR_INVALID, "no split for this kind or shape");
+    const int half = S / 2, cus = compute_units > 0 ? compute_units : 256;
+    auto valid = [&](int s) { return s <= max_split && half % s == 0 && N % (s >= 64 ? 1 : 64 / s) == 0; };
+    auto tasks = [&](int s) { return (long)N * s / 64; };
+    int pick = 0;
+    for (int s = 8; s <= max_split; s *= 2)
+        if (valid(s)) {
+            pick = s;  // (the largest valid one if none gets the lanes short enough)
+            if (half / s <= 72) break;
+        }
+    if (!pick) return fail(SPTMM_ERR_INVALID, "Wrong SPLIT Size: no split_k in 8..%d divides S/2 = %d with N = %d", max_split, half, N);
+    while (tasks(pick) < 2L * cus && valid(2 * pick) && half / (2 * pick) >= 8) pick *= 2;
+    return pick;
+}
+
 int sptmm_pack_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, void *out)
 {
     return guarded([&]() -> int {

@@ -352,3 +352,29 @@ def test_non_positive_shapes_are_refused_before_anything_is_read():
             assert L.sptmm_pack_ragged(C.c_void_p(P(W)), K, N, kind, 32, 8, C.c_void_p(P(out))) == -1
         assert L.sptmm_pack_i2s_bytes(K, N) == 0
         assert L.sptmm_pack_i2s(C.c_void_p(P(W)), K, N, C.c_void_p(P(out))) == -1
+
+
+def test_automatic_split_k_is_valid_and_follows_the_measured_rule():
+    """split_k = 0 in the upload calls: 30-70 entries per lane where the matrix is wide enough for two tasks per
+    compute unit, shorter lanes (down to 8 entries) where it is not; always a split the packers accept."""
+    want = {(sp.KIND_U16, 2560, 4096): 32, (sp.KIND_DELTA, 2560, 4096): 32, (sp.KIND_U16, 640, 1536): 64, (sp.KIND_U16, 2560, 1536): 16,
+            (sp.KIND_U16, 6912, 1536): 16, (sp.KIND_U16, 5120, 8320): 64, (sp.KIND_DELTA, 5120, 8320): 64, (sp.KIND_U16, 128, 4096): 256,
+            (sp.KIND_DELTA, 128, 4096): 64, (sp.KIND_U16, 2560, 4160): 32}
+    for (kind, N, S), split in want.items():
+        assert sp.choose_split_k(kind, N, S, 256) == split, (kind, N, S)
+    rng = np.random.default_rng(3)
+    for _ in range(300):
+        N = 16 * int(rng.integers(1, 900))
+        S = 2 * int(rng.integers(1, 5000))
+        for kind in (sp.KIND_U16, sp.KIND_DELTA):
+            try:
+                s = sp.choose_split_k(kind, N, S, int(rng.choice([0, 64, 256, 304])))
+            except sp.SptmmError as e:
+                assert e.code == -1 and all((S // 2) % x for x in (8, 16, 32, 64, 128, 256)[: 6 if kind == sp.KIND_U16 else 4])
+                continue
+            assert s in (8, 16, 32, 64, 128, 256)[: 6 if kind == sp.KIND_U16 else 4] and (S // 2) % s == 0 and N % max(1, 64 // s) == 0
+            n = sp.lib().sptmm_pack_u16_bytes(N, S, s) if kind == sp.KIND_U16 else sp.lib().sptmm_pack_delta_bytes(N, S, s, 8)
+            assert n > 0
+    for bad in ((sp.KIND_I2S, 64, 64), (sp.KIND_U16, 0, 64), (sp.KIND_U16, 64, 0), (sp.KIND_U16, 64, 31), (sp.KIND_U16, -16, 64)):
+        with pytest.raises(sp.SptmmError):
+            sp.choose_split_k(*bad)

@@ -152,6 +152,26 @@ def test_u16_special_inputs():
     w.free()
 
 
+@pytest.mark.parametrize("K,N,S", [(6912, 2560, 4096), (2560, 640, 1536), (6912, 128, 4096), (13824, 256, 8320)])
+def test_automatic_split_k(K, N, S, device):
+    """split_k = 0: the library picks (sptmm_choose_split_k for this device); the result is the same as with any split."""
+    W, pos, neg = matrix(K, N, S, dense=True)
+    cus = device["compute_units"]
+    ws = [sp.Weights.upload_u16(pos, neg, K, 0), sp.Weights.upload_delta(pos, neg, K, 0), sp.Weights.upload_dense(W, sp.KIND_U16, 0),
+          sp.Weights.upload_dense(W, sp.KIND_DELTA, 0), sp.Weights.upload_wide(W, sp.KIND_U16, 0), sp.Weights.upload_wide(W, sp.KIND_DELTA, 0)]
+    assert ws[0].info["split_k"] == sp.choose_split_k(sp.KIND_U16, N, S, cus)
+    assert ws[1].info["split_k"] == sp.choose_split_k(sp.KIND_DELTA, N, S, cus)
+    for M in (1, 4, 9):
+        X = x_i8(50 + M, M, K)
+        want = oracle.sptmm_i8_mt(X, pos, neg, 8)
+        for w in ws:
+            say("auto split", K, N, S, "kind", w.info["kind"], "ragged", w.info["ragged"], "k_tile", w.info["k_tile"], "split", w.info["split_k"], "M", M)
+            assert w.info["split_k"] in (8, 16, 32, 64, 128, 256)
+            assert (w.matmul(X) == want).all()
+    for w in ws:
+        w.free()
+
+
 def test_linearity_and_split_invariance_full_size():
     K, N, S = 6912, 2560, 4096
     _, pos, neg = matrix(K, N, S)
