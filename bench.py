@@ -100,6 +100,9 @@ def main():
     ap.add_argument("--steps", type=int, default=256, help="timed steps; one step = one launch of BATCH GEMVs")
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--reps", type=int, default=0,
+                    help="launches per timed loop of the legs (0: 1500, the headline shape's other encodings 4096); counter "
+                         "runs under a profiler, where every launch is serialised, use a few dozen")
     ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,cfg4",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, sync-each-call), "
                          "others (delta and i2s encodings at the headline shape), cfg1 (the same matrix at M=4), cfg2 (gap "
@@ -136,6 +139,7 @@ def main():
         return us, (time.perf_counter() - t0) * 1e3 / launches
 
     def time_encoding(w, act, Xh, m, n_cols, k_rows, reps=1500):
+        reps = a.reps or reps
         """One weights object at one activation shape: one GEMV per launch on the same stream every launch
         (cache-warm) and rotating over enough device copies to exceed the last-level cache (HBM-cold), and
         32 (or as many as there are copies) per launch, HBM-cold.  Best of two, microseconds per GEMV."""
@@ -144,14 +148,14 @@ def main():
         cps = [w] + [w.clone() for _ in range(ncp - 1)]
         cd = sp.DeviceBuffer(4 * m * n_cols * min(ncp, BATCH))
         nb = algorithmic_bytes(w.info["stream_bytes"], m, k_rows, n_cols, Xh.itemsize)
-        sp.measure_gemv(cps[:1], act, xd, m, cd, 200, 0, st)
+        sp.measure_gemv(cps[:1], act, xd, m, cd, min(200, reps), 0, st)
         warm = min(sp.measure_gemv(cps[:1], act, xd, m, cd, reps, 0, st) for _ in range(2))
         sp.measure_gemv(cps, act, xd, m, cd, 2 * ncp, 0, st)
         cold = min(sp.measure_gemv(cps, act, xd, m, cd, reps, 0, st) for _ in range(2))
         groups = [cps[i:i + BATCH] for i in range(0, ncp, BATCH) if len(cps[i:i + BATCH]) == min(ncp, BATCH)]
         for g in groups:
             sp.measure_gemv(g, act, xd, m, cd, 2 * len(g), 3, st)
-        per_group = max(8, 96 // len(groups))
+        per_group = max(8, min(96, reps) // len(groups))
         bat = min(sum(sp.measure_gemv(g, act, xd, m, cd, per_group * len(g), 3, st) for g in groups) / len(groups) for _ in range(2))
         for o in cps[1:] + [xd, cd]:
             o.free()
