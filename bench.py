@@ -169,20 +169,25 @@ def main():
         the library picks for the shape (sptmm_choose_split_k); the row's `split_k` says which."""
         Wm, p, n = lists if lists is not None else sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)
         rows = []
-        makers = (("u16", lambda: sp.Weights.upload_u16(p, n, k_rows, split)),
-                  ("delta", lambda: sp.Weights.upload_delta(p, n, k_rows, split)),
-                  ("i2s", lambda: sp.Weights.upload_i2s(Wm)))
+        # gap streams are packed for the number of activation rows they will meet: the GEMV stream (rows = 1) or the plain one
+        makers = (("u16", lambda m: sp.Weights.upload_u16(p, n, k_rows, split)),
+                  ("delta", lambda m: sp.Weights.upload_delta(p, n, k_rows, split, rows=m)),
+                  ("i2s", lambda m: sp.Weights.upload_i2s(Wm)))
         refs = {}
         for enc, mk in makers:
-            w = mk()
+            w = None
             for m in ms:
+                if w is None or (enc == "delta" and (m == 1) != (w.info["row_bytes"] == 1)):
+                    if w is not None:
+                        w.free()
+                    w = mk(m)
                 Xm = sp.make_x_i8(0xC0FFEE ^ m, m, k_rows)
                 got = w.matmul(Xm)
                 if m not in refs:
                     refs[m] = got
                     checks.append(("%s M=%d" % (label, m), Xm, p, n, got, s_nz))
                 r = {"shape": label, "K": k_rows, "N": n_cols, "S": s_nz, "M": m, "enc": enc, "split_k": w.info["split_k"],
-                     "bit_exact_across_encodings": bool((got == refs[m]).all())}
+                     "row_bytes": w.info["row_bytes"], "bit_exact_across_encodings": bool((got == refs[m]).all())}
                 r.update(time_encoding(w, 0, Xm, m, n_cols, k_rows))
                 rows.append(r)
             w.free()
@@ -249,7 +254,7 @@ def main():
 
     others = {}
     if "others" in legs:
-        for name, mk in (("delta8_split32", lambda: sp.Weights.upload_delta(pos, neg, K, SPLIT)),
+        for name, mk in (("delta8_split32", lambda: sp.Weights.upload_delta(pos, neg, K, SPLIT, rows=M)),
                          ("i2s", lambda: sp.Weights.upload_i2s(Wd))):
             ww = mk()
             assert (ww.matmul(X) == ref).all(), name

@@ -60,6 +60,8 @@ typedef struct sptmm_winfo {
     int ragged;      /* 1: built from a matrix whose columns differ in nonzeros (S is 0 then) */
     uint64_t nnz;    /* nonzeros of the whole matrix */
     int k_tile;      /* wide streams: rows per K-tile (0 for every other stream) */
+    int row_bytes;   /* 8-bit gap streams: bytes per row of the activation tile the visiting order was scheduled for,
+                      * 1 (sptmm_*_rows with rows = 1) or 4; 0 for every other stream */
 } sptmm_winfo;
 
 typedef struct sptmm_weights sptmm_weights; /* opaque; owns its device buffer */
@@ -110,6 +112,13 @@ int sptmm_delta_bits(const uint16_t *pos, const uint16_t *neg, int N, int S, int
 size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits);
 int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out);
 int sptmm_unpack_delta(const void *packed, int K, int N, int S, int split_k, int bits, uint16_t *pos, uint16_t *neg);
+/* The same stream with the visiting order of the 8-bit gaps chosen for calls with `rows` activation
+ * rows.  rows = 1: for an activation tile of ONE BYTE per row (int8, a single row: the GEMV of
+ * main.cu:556-594 at M = 1), where the gather address is the running row itself and the LDS bank of a
+ * row is (row / 4) mod 32; any other value: as sptmm_pack_delta (4-byte slots, bank = row mod 32).
+ * Size, layout and sptmm_unpack_delta are the same either way; every GEMV entry point serves either
+ * stream at any M, fastest at the M it was scheduled for.  No counterpart in the reference. */
+int sptmm_pack_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, int rows, void *out);
 
 /* Ragged matrices: any K x N matrix over {-1,0,+1} (column n at W + n*K), columns
  * free to differ in nonzeros and in their +1/-1 split -- what a quantised model
@@ -126,6 +135,8 @@ size_t sptmm_pack_ragged_bytes(const int8_t *W_colmajor, int K, int N, int kind,
                                int *n_min, int *n_max, uint64_t *nnz);
 int sptmm_pack_ragged(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int bits, void *out);
 int sptmm_unpack_ragged(const void *packed, int K, int N, int kind, int split_k, int bits, int8_t *W_colmajor);
+/* As sptmm_pack_ragged, gap streams scheduled for `rows` activation rows per call (see sptmm_pack_delta_rows). */
+int sptmm_pack_ragged_rows(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int bits, int rows, void *out);
 /* Seeded matrix with independent entries: +1 with probability p_pos, -1 with
  * p_neg (xorshift32 of macro.cuh:69-76 per column, state seed ^ 0x9E3779B9*(n+1);
  * entry = top 24 bits of the next state against the two thresholds). */
@@ -168,11 +179,16 @@ int sptmm_device_init(int device, sptmm_devinfo *out);
  * current device (ragged matrices: from the mean nonzeros per column). */
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
+/* Gap stream scheduled for calls with `rows` activation rows (sptmm_pack_delta_rows): rows = 1 is
+ * the stream for GEMVs (int8, M = 1); 0 = no preference (as sptmm_weights_upload_delta). */
+int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int rows, sptmm_weights **out);
 int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weights **out);
 /* Any ternary matrix -> device stream of the given kind (ragged u16 lists,
  * ragged gap stream, or i2s).  The GEMV entry points below serve it like any
  * other weights object. */
 int sptmm_weights_upload_dense(const int8_t *W_colmajor, int K, int N, int kind, int split_k, sptmm_weights **out);
+/* The same with a gap stream scheduled for `rows` activation rows per call (see sptmm_weights_upload_delta_rows). */
+int sptmm_weights_upload_dense_rows(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int rows, sptmm_weights **out);
 /* Any ternary matrix -> wide device stream (u16 lists or gap stream), K-tiled for this device's
  * LDS.  sptmm_gemv_i8 and sptmm_gemv_f16 (and the batched call) serve it with 16-row (8-row) tiles:
  * meant for M > 8 (M > 4 with fp16 rows); correct for any M.  No counterpart in the reference. */

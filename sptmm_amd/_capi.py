@@ -27,7 +27,8 @@ EXPORTS = [
     "sptmm_unpack_ragged", "sptmm_generate_ternary_iid", "sptmm_dense_from_i2s_words", "sptmm_weights_upload_dense",
     "sptmm_choose_split_k", "sptmm_wide_k_tile", "sptmm_pack_wide_bytes", "sptmm_pack_wide", "sptmm_unpack_wide", "sptmm_weights_upload_wide",
     "sptmm_device_init",
-    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta",
+    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_delta_rows", "sptmm_weights_upload_dense_rows",
+    "sptmm_pack_delta_rows", "sptmm_pack_ragged_rows",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
     "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_i8_batched", "sptmm_gemv_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
@@ -53,7 +54,7 @@ class DevInfo(C.Structure):
 class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
                 ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64),
-                ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int)]
+                ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int), ("row_bytes", C.c_int)]
 
 
 def lib_path() -> str:
@@ -179,13 +180,14 @@ def delta_bits(pos, neg, split_k) -> int:
     return _ck(lib().sptmm_delta_bits(_p(pos), _p(neg), N, 2 * half, split_k))
 
 
-def pack_delta(pos, neg, K, split_k, bits=None) -> tuple[np.ndarray, int]:
+def pack_delta(pos, neg, K, split_k, bits=None, rows=0) -> tuple[np.ndarray, int]:
+    """rows = 1: 8-bit gaps visited in the order scheduled for a tile of one byte per row (GEMV, int8, M = 1)."""
     N, half = pos.shape
     if bits is None:
         bits = delta_bits(pos, neg, split_k)
     n = lib().sptmm_pack_delta_bytes(N, 2 * half, split_k, bits)
     out = np.zeros(max(n, 1), np.uint8)
-    _ck(lib().sptmm_pack_delta(_p(pos), _p(neg), K, N, 2 * half, split_k, bits, _p(out)))
+    _ck(lib().sptmm_pack_delta_rows(_p(pos), _p(neg), K, N, 2 * half, split_k, bits, rows, _p(out)))
     return out[:n], bits
 
 
@@ -237,7 +239,7 @@ def dense_from_i2s_words(words: np.ndarray, K: int) -> np.ndarray:
     return W
 
 
-def pack_ragged(W: np.ndarray, kind: int, split_k: int, bits: int = 0):
+def pack_ragged(W: np.ndarray, kind: int, split_k: int, bits: int = 0, rows: int = 0):
     """Any ternary matrix W [N][K] -> (stream bytes, dict(bits, read_bytes, n_min, n_max, nnz))."""
     N, K = W.shape
     b, rb, lo, hi, nnz = C.c_int(bits), C.c_size_t(), C.c_int(), C.c_int(), C.c_uint64()
@@ -245,7 +247,7 @@ def pack_ragged(W: np.ndarray, kind: int, split_k: int, bits: int = 0):
     if not n:
         raise SptmmError(-1, lib().sptmm_last_error().decode())
     out = np.zeros(n, np.uint8)
-    _ck(lib().sptmm_pack_ragged(_p(W), K, N, kind, split_k, b.value, _p(out)))
+    _ck(lib().sptmm_pack_ragged_rows(_p(W), K, N, kind, split_k, b.value, rows, _p(out)))
     return out, {"bits": b.value, "read_bytes": rb.value, "n_min": lo.value, "n_max": hi.value, "nnz": nnz.value}
 
 
@@ -462,10 +464,11 @@ class Weights:
         return cls(h)
 
     @classmethod
-    def upload_delta(cls, pos, neg, K, split_k) -> "Weights":
+    def upload_delta(cls, pos, neg, K, split_k, rows=0) -> "Weights":
+        """rows: activation rows per call the gap stream is scheduled for (1: the GEMV stream, int8 M = 1; 0: no preference)."""
         N, half = pos.shape
         h = C.c_void_p()
-        _ck(lib().sptmm_weights_upload_delta(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(h)))
+        _ck(lib().sptmm_weights_upload_delta_rows(_p(pos), _p(neg), K, N, 2 * half, split_k, rows, C.byref(h)))
         return cls(h)
 
     @classmethod
@@ -476,11 +479,11 @@ class Weights:
         return cls(h)
 
     @classmethod
-    def upload_dense(cls, W: np.ndarray, kind: int, split_k: int = 32) -> "Weights":
-        """Any ternary matrix W [N][K] (columns free to differ in nonzeros) in the given encoding."""
+    def upload_dense(cls, W: np.ndarray, kind: int, split_k: int = 32, rows: int = 0) -> "Weights":
+        """Any ternary matrix W [N][K] (columns free to differ in nonzeros) in the given encoding; rows as in upload_delta."""
         N, K = W.shape
         h = C.c_void_p()
-        _ck(lib().sptmm_weights_upload_dense(_p(W), K, N, kind, split_k, C.byref(h)))
+        _ck(lib().sptmm_weights_upload_dense_rows(_p(W), K, N, kind, split_k, rows, C.byref(h)))
         return cls(h)
 
     @classmethod

@@ -23,6 +23,7 @@ struct sptmm_weights {
     int task_stride = 0, counts_bytes = 0;  // ragged streams
     int n_min = 0, n_max = 0;
     int index_shift = 0;  // u16 streams: fields are row << index_shift
+    bool byte_rows = false;  // 8-bit gap stream scheduled for a tile of one byte per row
     bool wide = false;    // wide stream (K-tiled, 16-byte slots): `wh` describes it
     WideHeader wh;
 };
@@ -140,6 +141,7 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.n_min = w->n_min;
     a.n_max = w->n_max;
     a.index_shift = w->index_shift;
+    a.byte_rows = w->byte_rows;
     a.ragged = w->info.ragged;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
@@ -213,8 +215,14 @@ int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, in
 
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out)
 {
+    return sptmm_weights_upload_delta_rows(pos, neg, K, N, S, split_k, 0, out);
+}
+
+int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int rows, sptmm_weights **out)
+{
     return guarded([&]() -> int {
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         if (int rc = check_shape(K, N, S)) return rc;
         if (int rc = resolve_split(SPTMM_KIND_DELTA, N, S, &split_k)) return rc;
         Geometry g;
@@ -222,11 +230,13 @@ int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, 
         int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
         if (bits < 0) return bits;
         std::vector<uint8_t> host(sptmm_pack_delta_bytes(N, S, split_k, bits));
-        if (int rc = sptmm_pack_delta(pos, neg, K, N, S, split_k, bits, host.data())) return rc;
+        if (int rc = sptmm_pack_delta_rows(pos, neg, K, N, S, split_k, bits, rows, host.data())) return rc;
         sptmm_weights *w = new (std::nothrow) sptmm_weights();
         if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
         w->info = sptmm_winfo{SPTMM_KIND_DELTA, K, N, S, split_k, bits, 0, 0, (uint64_t)S * N};
         w->geo = g;
+        w->byte_rows = bits == 8 && rows == 1;
+        w->info.row_bytes = bits == 8 ? (rows == 1 ? 1 : 4) : 0;
         return finish_upload(w, host, out);
     });
 }
@@ -249,8 +259,14 @@ int sptmm_weights_upload_i2s(const int8_t *W, int K, int N, sptmm_weights **out)
 
 int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int split_k, sptmm_weights **out)
 {
+    return sptmm_weights_upload_dense_rows(W, K, N, kind, split_k, 0, out);
+}
+
+int sptmm_weights_upload_dense_rows(const int8_t *W, int K, int N, int kind, int split_k, int rows, sptmm_weights **out)
+{
     return guarded([&]() -> int {
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         if (kind == SPTMM_KIND_I2S) return sptmm_weights_upload_i2s(W, K, N, out);
         if (int rc = resolve_split_dense(W, K, N, kind, &split_k)) return rc;
         int bits = 0, n_min = 0, n_max = 0;
@@ -259,7 +275,7 @@ int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int spli
         const size_t bytes = sptmm_pack_ragged_bytes(W, K, N, kind, split_k, &bits, &read_bytes, &n_min, &n_max, &nnz);
         if (!bytes) return SPTMM_ERR_INVALID;  // message set by the planner
         std::vector<uint8_t> host(bytes);
-        if (int rc = sptmm_pack_ragged(W, K, N, kind, split_k, bits, host.data())) return rc;
+        if (int rc = sptmm_pack_ragged_rows(W, K, N, kind, split_k, bits, rows, host.data())) return rc;
         sptmm_weights *w = new (std::nothrow) sptmm_weights();
         if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
         w->info = sptmm_winfo{kind, K, N, 0, split_k, bits, read_bytes, 1, nnz};
@@ -272,6 +288,8 @@ int sptmm_weights_upload_dense(const int8_t *W, int K, int N, int kind, int spli
         w->n_min = n_min;
         w->n_max = n_max;
         w->index_shift = kind == SPTMM_KIND_U16 ? ragged_index_shift(K) : 0;
+        w->byte_rows = kind == SPTMM_KIND_DELTA && bits == 8 && rows == 1;
+        w->info.row_bytes = kind == SPTMM_KIND_DELTA && bits == 8 ? (rows == 1 ? 1 : 4) : 0;
         return finish_upload(w, host, out);
     });
 }
@@ -355,7 +373,9 @@ struct FileHeader {
     uint32_t version;         // 2 (1: i2s tiles in the older lane order, column-major inside a tile; re-tiled on load)
     int32_t kind, K, N, S, split_k, delta_bits, ragged;
     int32_t half, L, G, W, n_lane, tasks;
-    int32_t task_stride, counts_bytes, n_min, n_max, index_shift;
+    int32_t task_stride, counts_bytes, n_min, n_max;
+    int32_t index_shift;      // u16 lists: fields are row << index_shift; 8-bit gap streams: 2 when the visiting order was scheduled for
+                              // tiles of one byte per row (LDS bank = (row >> 2) mod 32), else 0
     uint64_t nnz, read_bytes, stream_bytes;
     uint64_t fnv1a;           // of the header (this field zero) and the stream
 };
@@ -390,7 +410,8 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
         const Geometry &g = w->geo;
         h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = i.ragged;
         h.half = g.half, h.L = g.L, h.G = g.G, h.W = g.W, h.n_lane = g.n_lane, h.tasks = g.tasks;
-        h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max, h.index_shift = w->index_shift;
+        h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max;
+        h.index_shift = i.kind == SPTMM_KIND_DELTA ? (w->byte_rows ? 2 : 0) : w->index_shift;
         h.nnz = i.nnz, h.read_bytes = i.stream_bytes, h.stream_bytes = w->bytes;
         h.fnv1a = file_checksum(h, host);
         FILE *f = fopen(path, "wb");
@@ -428,13 +449,13 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
                     if (h.K <= 0 || h.N <= 0 || h.K % 16 || h.N % 16 || h.K + 64 > 65535 || make_ragged_geometry(h.N, h.split_k, max_split, &g) ||
                         h.n_min < 1 || h.n_max < h.n_min || h.n_max > 65535 || h.counts_bytes != (int)ragged_counts_bytes(g.tasks) ||
                         h.task_stride != (gaps ? 256 : 0) + 128 * esz * h.n_max ||
-                        h.index_shift != (gaps ? 0 : ragged_index_shift(h.K)))
+                        (gaps ? (h.index_shift != 0 && !(h.index_shift == 2 && h.delta_bits == 8)) : h.index_shift != ragged_index_shift(h.K)))
                         rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent ragged stream header", path);
                     else
                         want = (size_t)h.counts_bytes + (size_t)h.task_stride * g.tasks;
                 } else {
                     if (check_shape(h.K, h.N, h.S) || make_geometry(h.N, h.S, h.split_k, max_split, &g) ||
-                        h.index_shift != (gaps ? 0 : u16_index_shift(h.K)))
+                        (gaps ? (h.index_shift != 0 && !(h.index_shift == 2 && h.delta_bits == 8)) : h.index_shift != u16_index_shift(h.K)))
                         rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent stream header", path);
                     else
                         want = gaps ? sptmm_pack_delta_bytes(h.N, h.S, h.split_k, h.delta_bits) : sptmm_pack_u16_bytes(h.N, h.S, h.split_k);
@@ -480,7 +501,9 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         w->counts_bytes = h.counts_bytes;
         w->n_min = h.n_min;
         w->n_max = h.n_max;
-        w->index_shift = h.index_shift;
+        w->index_shift = h.kind == SPTMM_KIND_DELTA ? 0 : h.index_shift;
+        w->byte_rows = h.kind == SPTMM_KIND_DELTA && h.index_shift == 2;
+        w->info.row_bytes = h.kind == SPTMM_KIND_DELTA && h.delta_bits == 8 ? (w->byte_rows ? 1 : 4) : 0;
         return finish_upload(w, host, out);
     });
 }
@@ -503,7 +526,7 @@ int sptmm_gemv_batched(const sptmm_weights *const *ws, const void *const *X, voi
             if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
             const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
             if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
-                a.ragged != b.ragged || a.k_tile != b.k_tile || ws[0]->wide != ws[i]->wide ||
+                a.ragged != b.ragged || a.k_tile != b.k_tile || a.row_bytes != b.row_bytes || ws[0]->wide != ws[i]->wide ||
                 (ws[0]->wide && memcmp(&ws[0]->wh, &ws[i]->wh, sizeof(WideHeader)) != 0) || ws[0]->task_stride != ws[i]->task_stride ||
                 ws[0]->n_min != ws[i]->n_min)
                 return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);

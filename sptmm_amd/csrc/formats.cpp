@@ -268,7 +268,7 @@ void schedule(Domain &d)
 
 bool schedule_runs(RunDomain &d, int window)
 {
-    const int n = d.n, NL = d.lanes, mask = d.lanes - 1;  // lanes of the domain = banks it spreads over
+    const int n = d.n, NL = d.lanes, mask = d.lanes - 1, sh = d.shift;  // lanes of the domain = banks it spreads over
     struct Lane {
         std::vector<char> seen;   // visited entries
         int lo = 0, cur = -1;     // oldest entry not visited yet; row visited last
@@ -281,7 +281,7 @@ bool schedule_runs(RunDomain &d, int window)
         for (int i = 1; i < n; ++i)
             if (d.rows[l][i] - d.rows[l][i - 1] > 127) return false;
         for (int i = 0; i < n; ++i)
-            if (d.rows[l][i] < d.zero_row) ++demand[d.rows[l][i] & mask];
+            if (d.rows[l][i] < d.zero_row) ++demand[(d.rows[l][i] >> sh) & mask];
         lane[l].seen.assign(n, 0);
         d.order[l].assign(n, 0);
     }
@@ -290,7 +290,7 @@ bool schedule_runs(RunDomain &d, int window)
     struct Matcher {
         Lane *lane;
         RunDomain &d;
-        int cap = 1, mask = 31;
+        int cap = 1, mask = 31, sh = 0;
         int owners[32][32], count[32];
         bool tried[32];
         bool place(int l)
@@ -301,7 +301,7 @@ bool schedule_runs(RunDomain &d, int window)
                     lane[l].pick = i;
                     return true;
                 }
-                const int b = row & mask;
+                const int b = (row >> sh) & mask;
                 if (tried[b]) continue;
                 tried[b] = true;
                 if (count[b] < cap) {
@@ -320,6 +320,7 @@ bool schedule_runs(RunDomain &d, int window)
         }
     } m{lane, d};
     m.mask = mask;
+    m.sh = sh;
 
     double credit = 0.0;
     for (int step = 0; step < n; ++step) {
@@ -352,7 +353,7 @@ bool schedule_runs(RunDomain &d, int window)
             }
             if (L.cand.empty()) return false;  // cannot happen while the sorted gaps fit; kept as a guard
             std::stable_sort(L.cand.begin(), L.cand.end(), [&](int x, int y) {
-                const int dx = r[x] >= d.zero_row ? -1 : demand[r[x] & mask], dy = r[y] >= d.zero_row ? -1 : demand[r[y] & mask];
+                const int dx = r[x] >= d.zero_row ? -1 : demand[(r[x] >> sh) & mask], dy = r[y] >= d.zero_row ? -1 : demand[(r[y] >> sh) & mask];
                 return dx > dy;
             });
         }
@@ -370,13 +371,13 @@ bool schedule_runs(RunDomain &d, int window)
             if (!placed[l]) {  // no bank with room: join the least loaded one
                 int best = L.cand[0];
                 for (int i : L.cand)
-                    if (load[d.rows[l][i] & mask] < load[d.rows[l][best] & mask]) best = i;
+                    if (load[(d.rows[l][i] >> sh) & mask] < load[(d.rows[l][best] >> sh) & mask]) best = i;
                 L.pick = best;
-                ++load[d.rows[l][best] & mask];
+                ++load[(d.rows[l][best] >> sh) & mask];
             }
             L.seen[L.pick] = 1;
             L.cur = d.rows[l][L.pick];
-            if (L.cur < d.zero_row) --demand[L.cur & mask];
+            if (L.cur < d.zero_row) --demand[(L.cur >> sh) & mask];
             d.order[l][step] = (uint16_t)L.cur;
             while (L.lo < n && L.seen[L.lo]) ++L.lo;
         }
@@ -554,13 +555,14 @@ size_t sptmm_pack_delta_bytes(int N, int S, int split_k, int bits)
 
 namespace sptmm {
 
-bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint16_t> (&rows)[2][64])
+bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint16_t> (&rows)[2][64], int bank_shift)
 {
     for (int sign = 0; sign < 2; ++sign)
         for (int h = 0; h < 2; ++h) {
             RunDomain d;
             d.n = n;
             d.zero_row = zero_row;
+            d.shift = bank_shift;
             for (int l = 0; l < 32; ++l) d.rows[l] = rows[sign][32 * h + l];
             if (!schedule_runs(d)) return false;
             for (int l = 0; l < 32; ++l) {
@@ -577,7 +579,7 @@ bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint
 
 extern "C" {
 
-static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int K, int N, int S, int split_k, int bits)
+static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int K, int N, int S, int split_k, int bits, int bank_shift = 0)
 {
     if (int rc = check_shape(K, N, S)) return rc;
     Geometry g;
@@ -601,7 +603,7 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
                     const uint16_t *lst = (sign ? neg : pos) + (size_t)(t * g.G + lane / g.L) * g.half + (size_t)(lane % g.L) * g.n_lane;
                     rows[sign][lane].assign(lst, lst + g.n_lane);
                 }
-            if (!write_task_runs8(base + (size_t)t * task_bytes, g.n_lane, K, rows)) bad[t * g.G] = 1;
+            if (!write_task_runs8(base + (size_t)t * task_bytes, g.n_lane, K, rows, bank_shift)) bad[t * g.G] = 1;
         });
         for (int c = 0; c < N; ++c)
             if (bad[c]) return fail(SPTMM_ERR_INVALID, "column %d: a gap does not fit 8 bits (signed)", c);
@@ -645,7 +647,13 @@ static int delta_walk(bool pack, void *packed, uint16_t *pos, uint16_t *neg, int
 
 int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, void *out)
 {
+    return sptmm_pack_delta_rows(pos, neg, K, N, S, split_k, bits, 0, out);
+}
+
+int sptmm_pack_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int bits, int rows, void *out)
+{
     return guarded([&]() -> int {
+        if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         // shape first: the scan below trusts N and S
         if (int rc = check_shape(K, N, S)) return rc;
         Geometry g;
@@ -653,7 +661,7 @@ int sptmm_pack_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int
         if (!out || !pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
         for (size_t i = 0, n = (size_t)N * g.half; i < n; ++i)
             if (pos[i] >= K || neg[i] >= K) return fail(SPTMM_ERR_INVALID, "row index out of range");
-        return delta_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k, bits);
+        return delta_walk(true, out, (uint16_t *)pos, (uint16_t *)neg, K, N, S, split_k, bits, rows == 1 ? 2 : 0);
     });
 }
 

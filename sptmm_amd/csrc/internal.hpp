@@ -106,13 +106,14 @@ void schedule(Domain &d);
 struct RunDomain {
     int n = 0, zero_row = 0;
     int lanes = 32;  // lanes scheduled together = banks (row mod lanes) they are spread over; 16 for the wide tiles
+    int shift = 0;   // bank = (row >> shift) mod lanes: 2 for tiles of one byte per row
     std::vector<uint16_t> rows[32];
     std::vector<uint16_t> order[32];
 };
-bool schedule_runs(RunDomain &d, int window = 8);
+bool schedule_runs(RunDomain &d, int window = 16);  // (window 8: 1.30 LDS passes per step on the headline matrix, 16: 1.24, 24: 1.25)
 // One task of an 8-bit gap stream (header + rounds at `task`): rows[sign][lane] = what the lane
 // visits, ascending, n each.  False when a sorted gap exceeds 127.
-bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint16_t> (&rows)[2][64]);
+bool write_task_runs8(uint8_t *task, int n, int zero_row, const std::vector<uint16_t> (&rows)[2][64], int bank_shift = 0);
 
 // Geometry of a ragged stream (tasks carry their own entry count): as
 // make_geometry, with half = n_lane = 0.
@@ -152,6 +153,7 @@ struct GemvArgs {
     int n_min, n_max;   // smallest / largest per-task entry count
     int compute_units;
     int lds_limit;
+    int byte_rows = 0;    // 8-bit gap stream scheduled for a tile of one byte per row (int8, one activation row)
     int quant = 0;        // 1 / 2: X holds fp16 / bf16 rows, quantised to int8 in the kernel; C receives floats
     float w_scale = 1.f;  // quantising launches: factor applied to every output
     // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each

@@ -21,6 +21,12 @@ typedef unsigned int u32;
 // ------------------------------------------------------------------ helpers
 template <typename Act> struct Acc { typedef float type; };
 template <> struct Acc<int8_t> { typedef int type; };
+// int8 activations kept as they are, one byte per row index, in the tile of a single activation row
+// (gap streams whose visiting order was scheduled for such a tile: LDS bank = (row / 4) mod 32).
+// The gather address is the running row itself and the tile is a quarter of the int32 one.
+struct i8row { int8_t v; };
+template <> struct Acc<i8row> { typedef int type; };
+template <typename Act> constexpr bool is_byte_rows() { return std::is_same<Act, i8row>::value; }
 
 // Bytes one row index occupies in the LDS activation tile.  Every layout keeps
 // "dword address mod 32 == row index mod 32" at 4 bytes per index, which is the
@@ -28,7 +34,8 @@ template <> struct Acc<int8_t> { typedef int type; };
 // of a half-wavefront on 32 different LDS banks.
 template <typename Act, int MT> __host__ __device__ constexpr int slot_bytes()
 {
-    return sizeof(Act) == 1 ? (MT == 1 ? 4 : MT)        // int8: one int32 (M=1), or MT packed bytes
+    return is_byte_rows<Act>() ? 1                      // int8, one row, one byte per index
+           : sizeof(Act) == 1 ? (MT == 1 ? 4 : MT)      // int8: one int32 (M=1), or MT packed bytes
            : sizeof(Act) == 2 ? (MT == 1 ? 4 : 2 * MT)  // fp16: one fp32 (M=1), or MT halves
                               : 4 * MT;                 // fp32
 }
@@ -118,8 +125,8 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
     }
 
     // What one slot of the tile holds (all MT rows of one index), as read from LDS.
-    typedef typename std::conditional<sizeof(Act) == 1, Vec<u32, NW>,
-                                      typename std::conditional<sizeof(Act) == 2 && (MT > 1), Vec<_Float16, MT>, Vec<float, MT>>::type>::type Raw;
+    typedef typename std::conditional<is_byte_rows<Act>(), Vec<int8_t, 1>, typename std::conditional<sizeof(Act) == 1, Vec<u32, NW>,
+                                      typename std::conditional<sizeof(Act) == 2 && (MT > 1), Vec<_Float16, MT>, Vec<float, MT>>::type>::type>::type Raw;
 
     // the slot at byte offset `addr` of the tile
     static __device__ __forceinline__ Raw load(const unsigned char *lds, u32 addr) { return *reinterpret_cast<const Raw *>(lds + addr); }
@@ -194,18 +201,31 @@ template <int MODE> struct Flavour {
 };
 constexpr int RAGGED_PREAMBLE = 16;  // {magic, tasks, n_max, n_min} in front of the u16 count table
 
-// run += sign-extended byte B of d, in one SDWA add
+// run += sign-extended byte B of d, in one SDWA add.  The sum goes to a register of its own: with byte rows
+// it is the gather address as it stands, and an add in place would cost a copy per entry.
 template <int B> __device__ __forceinline__ void add_signed_byte(u32 &run, u32 d)
 {
+    u32 next;
     if constexpr (B == 0)
-        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:DWORD" : "+v"(run) : "v"(d));
+        asm("v_add_u32_sdwa %0, sext(%1), %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:DWORD" : "=v"(next) : "v"(d), "v"(run));
     else if constexpr (B == 1)
-        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:DWORD" : "+v"(run) : "v"(d));
+        asm("v_add_u32_sdwa %0, sext(%1), %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:DWORD" : "=v"(next) : "v"(d), "v"(run));
     else if constexpr (B == 2)
-        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2 src1_sel:DWORD" : "+v"(run) : "v"(d));
+        asm("v_add_u32_sdwa %0, sext(%1), %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2 src1_sel:DWORD" : "=v"(next) : "v"(d), "v"(run));
     else
-        asm("v_add_u32_sdwa %0, sext(%1), %0 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3 src1_sel:DWORD" : "+v"(run) : "v"(d));
+        asm("v_add_u32_sdwa %0, sext(%1), %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3 src1_sel:DWORD" : "=v"(next) : "v"(d), "v"(run));
+    run = next;
 }
+
+// the byte at an absolute LDS address
+typedef __attribute__((address_space(3))) const unsigned char *lds_ptr;
+template <class Raw> __device__ __forceinline__ Raw lds_byte(u32 addr)
+{
+    Raw r;
+    r.v[0] = *reinterpret_cast<__attribute__((address_space(3))) const int8_t *>((lds_ptr)(size_t)addr);
+    return r;
+}
+__device__ __forceinline__ u32 lds_address(const unsigned char *p) { return (u32)(size_t)(lds_ptr)p; }
 
 // `run` is the current row of a gap stream: the row index itself with 8-bit gaps,
 // the byte offset of the row's slot in the tile with 16-bit gaps.  fetch() turns
@@ -215,7 +235,21 @@ template <class S, int MODE, bool PRE, int NBYTES>
 __device__ __forceinline__ void fetch(const unsigned char *lds, u32 d, u32 &run, typename S::Raw *r)
 {
     constexpr int SH = ilog2(S::SLOT);
-    if constexpr (Flavour<MODE>::GAP8) {
+    if constexpr (Flavour<MODE>::GAP8 && S::SLOT == 1) {
+        // byte rows: `run` is the LDS address of the row's byte itself (the tile's own address is in it)
+        add_signed_byte<0>(run, d);
+        r[0] = lds_byte<typename S::Raw>(run);
+        if constexpr (NBYTES > 1) {
+            add_signed_byte<1>(run, d);
+            r[1] = lds_byte<typename S::Raw>(run);
+        }
+        if constexpr (NBYTES > 2) {
+            add_signed_byte<2>(run, d);
+            r[2] = lds_byte<typename S::Raw>(run);
+            add_signed_byte<3>(run, d);
+            r[3] = lds_byte<typename S::Raw>(run);
+        }
+    } else if constexpr (Flavour<MODE>::GAP8) {
         add_signed_byte<0>(run, d);
         r[0] = S::load(lds, run << SH);
         if constexpr (NBYTES > 1) {
@@ -353,7 +387,9 @@ template <typename Act, int MT> struct Stager {
     static __device__ __forceinline__ void store(unsigned char *lds, int item, const uint4 (&r)[NLOAD])
     {
         uint4 *t = reinterpret_cast<uint4 *>(lds);
-        if constexpr (sizeof(Act) == 1 && MT == 1) {  // 16 bytes -> 16 sign-extended dwords
+        if constexpr (is_byte_rows<Act>()) {
+            t[item] = r[0];
+        } else if constexpr (sizeof(Act) == 1 && MT == 1) {  // 16 bytes -> 16 sign-extended dwords
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 int d = (int)comp(r[0], j);
@@ -772,6 +808,7 @@ struct ListsBody {
                 const unsigned short *rs = reinterpret_cast<const unsigned short *>(tb);
                 runp = (u32)rs[lane] << (Fl::GAP8 ? 0 : SH);
                 runq = (u32)rs[64 + lane] << (Fl::GAP8 ? 0 : SH);
+                if constexpr (is_byte_rows<Act>()) runp += lds_address(smem), runq += lds_address(smem);
             }
             if constexpr (VAR) {
                 n_lane = __builtin_amdgcn_readfirstlane(n_ahead);
@@ -1068,6 +1105,9 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             }
         }
     }
+    // byte rows, batched: the tile is a quarter of the others' and the chip is filled along blockIdx.z; the largest
+    // workgroup does best (headline shape, 32 GEMVs per launch: 5 wavefronts 77 %, 8 wavefronts 79 % of HBM peak)
+    if (is_byte_rows<Act>() && a.batch) wpb = max_waves / a.W * a.W;
     if (tune_wpb > 0 && tune_wpb <= max_waves && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
@@ -1187,7 +1227,11 @@ template <int MODE, bool PRE, bool VAR>
 static int launch_lists_a(const GemvArgs &a, ActType act, hipStream_t st)
 {
     switch (act) {
-    case ACT_I8: return launch_lists_m<int8_t, MODE, PRE, VAR>(a, st);
+    case ACT_I8:
+        if constexpr (MODE == 1) {
+            if (a.byte_rows && a.M == 1 && !a.quant) return launch_lists_t<i8row, 1, MODE, PRE, VAR>(a, st);
+        }
+        return launch_lists_m<int8_t, MODE, PRE, VAR>(a, st);
     case ACT_F16: return launch_lists_m<_Float16, MODE, PRE, VAR>(a, st);
     case ACT_F32: return launch_lists_m<float, MODE, PRE, VAR>(a, st);
     }

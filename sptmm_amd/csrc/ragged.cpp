@@ -27,6 +27,7 @@ namespace {
 struct RaggedPlan {
     Geometry g;
     int K = 0, kind = 0, bits = 0, esz = 2, hdr = 0, shift = 0;
+    int bank_shift = 0;  // 8-bit gap streams: LDS bank = (row >> bank_shift) mod 32 (2: tiles of one byte per row)
     std::vector<std::vector<uint16_t>> rows[2];  // [sign][column]: ascending row lists
     std::vector<int> n_task;
     int n_min = 0, n_max = 0;
@@ -213,7 +214,7 @@ void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
                 for (int i = 0; i < n; ++i) r[i] = first + i < cnt ? e[first + i] : (uint16_t)pl.K;
             }
         if (pl.esz == 1) {
-            write_task_runs8(t, n, pl.K, rows);  // the plan has checked that every gap fits
+            write_task_runs8(t, n, pl.K, rows, pl.bank_shift);  // the plan has checked that every gap fits
         } else {
             for (int sign = 0; sign < 2; ++sign)
                 for (int lane = 0; lane < 64; ++lane) {
@@ -293,9 +294,16 @@ size_t sptmm_pack_ragged_bytes(const int8_t *W, int K, int N, int kind, int spli
 
 int sptmm_pack_ragged(const int8_t *W, int K, int N, int kind, int split_k, int bits, void *out)
 {
+    return sptmm_pack_ragged_rows(W, K, N, kind, split_k, bits, 0, out);
+}
+
+int sptmm_pack_ragged_rows(const int8_t *W, int K, int N, int kind, int split_k, int bits, int rows, void *out)
+{
     return guarded([&]() -> int {
+        if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         RaggedPlan pl;
         if (int rc = ragged_plan(W, K, N, kind, split_k, bits, &pl)) return rc;
+        pl.bank_shift = rows == 1 ? 2 : 0;
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
         memset(out, 0, pl.counts_bytes + pl.stride * pl.g.tasks);
         if (kind == SPTMM_KIND_U16)

@@ -318,7 +318,8 @@ int main(int argc, char **argv)
     }
     if (f.row_split_delta2 > 0) {
         sptmm_weights *w = nullptr;
-        CHECK_SPTMM(sptmm_weights_upload_delta(pos.data(), neg.data(), K, N, S, (int)f.row_split_delta2, &w));
+        // the gap stream is packed for the number of activation rows of this run (M = 1 with int8 rows: the GEMV stream)
+        CHECK_SPTMM(sptmm_weights_upload_delta_rows(pos.data(), neg.data(), K, N, S, (int)f.row_split_delta2, act == 0 ? M : 0, &w));
         run("sptmm-delta", w, true);
     }
     if (f.i2s) {

@@ -195,16 +195,23 @@ def slot_offset(n_lane, esz, sign, lane, j):
     raise AssertionError
 
 
+@pytest.mark.parametrize("rows", [0, 1, 4])
 @pytest.mark.parametrize("K,N,S,split", [(2560, 16, 1536, 32), (6912, 16, 4096, 64), (6912, 16, 4160, 16), (2560, 16, 1536, 8)])
-def test_delta_8bit_lanes_walk_their_own_run_in_a_bank_friendly_order(K, N, S, split):
+def test_delta_8bit_lanes_walk_their_own_run_in_a_bank_friendly_order(K, N, S, split, rows):
     """Each lane visits exactly the contiguous run of the sorted list the reference's gaps describe
     (main.cu:376-394: gap i = row i - row i-1), in an order whose steps fit a signed byte, and the 32
-    lanes of a half-wavefront mostly sit on 32 different banks (row mod 32)."""
+    lanes of a half-wavefront mostly sit on 32 different banks: row mod 32 for tiles of four bytes per
+    row, (row / 4) mod 32 for the one-byte-per-row tile of streams packed with rows = 1."""
     _, pos, neg = sp.generate_ternary(K, N, S)
     d_ref, wrapped = oracle.delta8(pos)
     assert wrapped == 0
-    pk, bits = sp.pack_delta(pos, neg, K, split)
+    pk, bits = sp.pack_delta(pos, neg, K, split, rows=rows)
     assert bits == 8
+    if rows != 1:  # any hint but 1 is the plain stream
+        assert (pk == sp.pack_delta(pos, neg, K, split)[0]).all()
+    p2, n2 = sp.unpack_delta(pk, K, N, S, split, 8)  # the visiting order does not change what the stream holds
+    assert (p2 == pos).all() and (n2 == neg).all()
+    bank_shift = 2 if rows == 1 else 0
     L, G = min(split, 64), 64 // min(split, 64)
     n_lane = (S // 2) // split
     task_bytes = 256 + 128 * n_lane
@@ -225,7 +232,7 @@ def test_delta_8bit_lanes_walk_their_own_run_in_a_bank_friendly_order(K, N, S, s
             walks = np.array(walks)
             for h in range(2):
                 for j in range(n_lane):
-                    passes += np.bincount(walks[32 * h:32 * h + 32, j] & 31, minlength=32).max()
+                    passes += np.bincount((walks[32 * h:32 * h + 32, j] >> bank_shift) & 31, minlength=32).max()
                     slots += 1
     # sorted order needs ~3.5 passes per step; the schedule must stay well below 2
     assert passes <= 1.45 * slots, (passes / slots)

@@ -141,6 +141,48 @@ def test_gap_stream_lanes_visit_their_run_then_the_zero_row():
                 assert gaps[0] == 0 and sorted(walk) == want
 
 
+@pytest.mark.parametrize("split", [8, 16, 32, 64])
+def test_gap_stream_for_single_rows_holds_the_same_matrix_on_other_banks(split):
+    """rows = 1: the same runs per lane, visited in an order that spreads a half-wavefront over the banks
+    (row / 4) mod 32 of a tile with one byte per row; size, counts and what unpacks are unchanged."""
+    K, N = 2560, 32
+    for W in (sp.generate_ternary_iid(K, N, 17, 0.3, 0.3), special_matrix(K, N)):
+        plain, inf0 = sp.pack_ragged(W, DELTA, split)
+        packed, inf = sp.pack_ragged(W, DELTA, split, rows=1)
+        assert inf == inf0 and len(packed) == len(plain)  # (the special matrix takes 16-bit gaps: sorted order either way)
+        assert (sp.unpack_ragged(packed, K, N, DELTA, split, inf["bits"]) == W).all()
+        assert (sp.pack_ragged(W, DELTA, split, rows=4)[0] == plain).all()
+    # a matrix with independent entries: count the LDS passes of the walks on both bank functions
+    W = sp.generate_ternary_iid(K, N, 17, 0.3, 0.3)
+    tasks, table = N // (64 // split), -(-(16 + 2 * (N // (64 // split))) // 256) * 256
+    res = {}
+    for rows in (0, 1):
+        packed, inf = sp.pack_ragged(W, DELTA, split, rows=rows)
+        stride = 256 + 128 * inf["n_max"]
+        for shift in (0, 2):
+            passes = slots = 0
+            for t in range(tasks):
+                task = packed[table + t * stride:table + (t + 1) * stride]
+                n = int(packed[16 + 2 * t:][:2].view(np.uint16)[0])
+                for sign in (0, 1):
+                    walks = np.empty((64, n), int)
+                    for lane in range(64):
+                        first = int(task[sign * 128 + 2 * lane: sign * 128 + 2 * lane + 2].view(np.uint16)[0])
+                        gaps = task[[256 + slot_offset(n, 1, sign, lane, j) for j in range(n)]].view(np.int8).astype(int)
+                        walks[lane] = first + np.cumsum(gaps)
+                    for h in range(2):
+                        for j in range(n):
+                            real = walks[32 * h:32 * h + 32, j]
+                            real = real[real < K]  # the zero row is one address for every lane: no conflict
+                            if shift:
+                                real = np.unique(real >> 2) << 2  # lanes on one dword of the byte tile are served together
+                            passes += max(1, np.bincount((real >> shift) & 31, minlength=32).max()) if len(real) else 1
+                            slots += 1
+            res[rows, shift] = passes / slots
+    assert res[1, 2] <= 1.6 and res[0, 0] <= 1.6, res      # each stream on the banks it was scheduled for
+    assert res[1, 0] > res[1, 2] + 0.5 and res[0, 2] > res[0, 0] + 0.5, res  # and clearly worse on the other tile
+
+
 def test_sparse_matrix_takes_16_bit_gaps_and_8_bit_request_fails():
     K, N = 6912, 32
     W = sp.generate_ternary_iid(K, N, 5, 0.01, 0.01)
