@@ -46,7 +46,7 @@ def pct(nbytes, us):
     return round(100.0 * nbytes / us / 1e3 / PEAK_GBPS, 2)
 
 
-def cpu_baseline(sp_lists, gpu_headline, checks, budget_s=12.0):
+def cpu_baseline(sp_lists, gpu_headline, checks, dense_w=None, budget_s=12.0):
     """The oracle's gather-sum (a port of main.cu:577-593) on the host cores, bounded sample; and the
     oracle as checker of what the GPU legs computed."""
     import numpy as np
@@ -73,6 +73,16 @@ def cpu_baseline(sp_lists, gpu_headline, checks, budget_s=12.0):
                 break
         res[threads] = (el / reps * 1e6, reps)
     us, reps = res[cores]
+    # for context: the dense int8 product of the same matrix (single thread), and that it gives the same numbers
+    dense_us = None
+    if dense_w is not None:
+        t = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            dense = oracle.dense_i8(X, dense_w)
+            t.append(time.perf_counter() - t0)
+        assert (dense == want).all()
+        dense_us = round(sorted(t)[1] * 1e6, 1)
     bad = []
     for label, Xc, p, n, got, s_nz in checks:
         if Xc.dtype == np.int8:
@@ -86,7 +96,7 @@ def cpu_baseline(sp_lists, gpu_headline, checks, budget_s=12.0):
         "value": round(us, 2), "unit": "us/GEMV", "cores": cores, "cores_available": have, "kind": "port",
         "sample": "%d full GEMVs of the same W and X (oracle gather-sum over u16 lists, %d pthreads of the %d cores "
                   "this process may use); single thread: %.1f us/GEMV over %d GEMVs" % (reps, cores, have, res[1][0], res[1][1]),
-        "value_1core": round(res[1][0], 2),
+        "value_1core": round(res[1][0], 2), "dense_int8_1core_us": dense_us,
         "gbps": round(algorithmic_bytes(2 * S * N, M, K, N) / us / 1e3, 2),
         "gpu_headline_equals_oracle": headline_ok,
         "gpu_results_checked_against_oracle": len(checks) + 1,
@@ -352,7 +362,7 @@ def main():
         out["roofline"]["streaming_read_ceiling"] = ceiling
         out["roofline"]["frac_of_streaming_read"] = round(gbps / ceiling["gbps"], 4)
     if not a.no_cpu:
-        out["cpu_baseline"] = cpu_baseline((pos, neg), ref, checks)
+        out["cpu_baseline"] = cpu_baseline((pos, neg), ref, checks, Wd)
     w.free()
     print(json.dumps(out, ensure_ascii=False))
 

@@ -32,3 +32,23 @@ def test_json_line_has_the_contract_keys():
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3 and 0.3 < rf["frac"] < 1.0
     assert abs(j["value"] * 32 - rf["launch_us"]) < 0.05 * rf["launch_us"]
     assert 0.5 < rf["frac_of_streaming_read"] < 1.3
+    side = json.load(open(os.path.join(ROOT, "profiles", "traffic_lists_kernel_batched_i8_u16_cfg0.json")))
+    assert rf["traffic"] == side["traffic_bytes_per_launch"] and rf["traffic_source"]["measured_at_commit"] == side["measured_at_commit"]
+    assert rf["algorithmic_bytes_per_launch"] == side["algorithmic_bytes_per_launch"]
+
+
+def test_traffic_sidecar_is_consistent():
+    """roofline.traffic comes from a counter run kept in profiles/: the file names its commit and commands, and its
+    bytes follow from its own counter readings and scale factors."""
+    side = json.load(open(os.path.join(ROOT, "profiles", "traffic_lists_kernel_batched_i8_u16_cfg0.json")))
+    for k in ("kernel", "workload", "measured_at_commit", "commands", "fetch_size_kib_per_dispatch", "write_size_kib_per_dispatch",
+              "copy_kernel", "scale", "traffic_bytes_per_launch", "algorithmic_bytes_per_launch"):
+        assert k in side, k
+    cp = side["copy_kernel"]
+    assert abs(cp["bytes_read"] / 1024 / cp["fetch_size_kib_per_dispatch"] - side["scale"]["fetch_size"]) < 0.01
+    assert abs(cp["bytes_written"] / 1024 / cp["write_size_kib_per_dispatch"] - side["scale"]["write_size"]) < 0.01
+    want = (side["fetch_size_kib_per_dispatch"] * side["scale"]["fetch_size"] + side["write_size_kib_per_dispatch"] * side["scale"]["write_size"]) * 1024
+    assert abs(side["traffic_bytes_per_launch"] - want) <= 1024
+    assert side["algorithmic_bytes_per_launch"] == 32 * (2 * 4096 * 2560 + 6912 + 4 * 2560)
+    assert 0.98 < side["traffic_bytes_per_launch"] / side["algorithmic_bytes_per_launch"] < 1.05
+    assert all("bench.py" in c and c.startswith("rocprofv3 --pmc") for c in side["commands"])
