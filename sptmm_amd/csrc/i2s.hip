@@ -238,7 +238,7 @@ __device__ __forceinline__ void i2s_mfma_body(const I2sParams &p, unsigned char 
         const int g = blockIdx.x * CT + c;
         wbase[c] = p.w + (size_t)(g < groups ? g : groups - 1) * p.rounds * 64;
     }
-    constexpr int DEPTH = CT >= 4 ? 3 : 4;          // rounds in flight per wavefront
+    constexpr int DEPTH = CT >= 8 ? 2 : CT >= 4 ? 3 : 4;  // rounds in flight per wavefront
     const int T = (p.rounds + waves - 1) / waves;   // steps every wavefront makes; step t of this one is round wave + t*waves
 
     v4i D[CT], D1 = {0, 0, 0, 0};
@@ -404,16 +404,17 @@ static int launch_i2s_mfma(const GemvArgs &a, hipStream_t st)
     const int rows = a.M < 16 ? a.M : 16, xj = (rows + 3) / 4;  // loads of X rows per round: four rows each
     // Column tiles per wavefront and wavefronts per workgroup, measured on MI355X (K=6912 N=2560 and K=13824
     // N=5120, 1 to 16 rows).  A batched launch fills the chip along blockIdx.z and does best with the most
-    // reuse of X: 4 tiles, 4 wavefronts.  A lone launch needs its workgroups to cover the compute units
-    // first: the most tiles that still leave ~160 workgroups, 8 wavefronts each.
+    // reuse of X: 4 tiles, 4 wavefronts -- 8 tiles from nine rows on, where X traffic from L2 still sets the time
+    // (K=13824 N=5120, 16 rows, 32 GEMVs per launch: 3.36 -> 3.01 us per GEMV; 8 rows: level).  A lone launch needs
+    // its workgroups to cover the compute units first: the most tiles that still leave ~160 workgroups, 8 wavefronts each.
     int ct = 1, waves = 8;
     if (a.batch >= 4) {
-        ct = 4;
+        ct = xj >= 3 ? 8 : 4;
         waves = 4;
     } else {
         while (ct < 4 && groups / (2 * ct) >= 160) ct *= 2;
     }
-    if (tune_ct == 1 || tune_ct == 2 || tune_ct == 4) ct = tune_ct;
+    if (tune_ct == 1 || tune_ct == 2 || tune_ct == 4 || (tune_ct == 8 && xj >= 2)) ct = tune_ct;
     if (waves > rounds) waves = rounds;
     if (tune_waves > 0 && tune_waves <= 8) waves = tune_waves;
 #define I2S_CASE(XJ, CT) \
@@ -422,6 +423,7 @@ static int launch_i2s_mfma(const GemvArgs &a, hipStream_t st)
     I2S_CASE(2, 1); I2S_CASE(2, 2); I2S_CASE(2, 4);
     I2S_CASE(3, 1); I2S_CASE(3, 2); I2S_CASE(3, 4);
     I2S_CASE(4, 1); I2S_CASE(4, 2); I2S_CASE(4, 4);
+    I2S_CASE(2, 8); I2S_CASE(3, 8); I2S_CASE(4, 8);
 #undef I2S_CASE
     return fail(SPTMM_ERR_INVALID, "no i2s kernel for %d rows", a.M);
 }

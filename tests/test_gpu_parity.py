@@ -551,6 +551,30 @@ def test_batched_launch_equals_single_launches(kind, M, count):
     st.destroy()
 
 
+@pytest.mark.parametrize("M,count", [(9, 4), (16, 5), (20, 4), (3, 6)])
+def test_i2s_batched_launch_column_tiles_past_the_last_group(M, count):
+    """From four GEMVs per launch the matrix-unit kernel gives a wavefront 4 column tiles (8 from nine rows on);
+    43 groups of 16 columns leave the last workgroup with tiles past the end, and 20 rows take two row tiles."""
+    K, N, S = 2560, 688, 1536
+    W, pos, neg = matrix(K, N, S, dense=True)
+    base = sp.Weights.upload_i2s(W)
+    ws = [base] + [base.clone() for _ in range(count - 1)]
+    Xs = [x_i8(9500 + i, M, K) for i in range(count)]
+    xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
+    cb = [sp.DeviceBuffer(4 * M * N) for _ in range(count)]
+    for c in cb:
+        c.fill(0xFF)
+    say("i2s batched", "M", M, "count", count)
+    st = sp.Stream()
+    sp.gemv_i8_batched(ws, xb, cb, M, st)
+    st.sync()
+    for i in range(count):
+        assert (cb[i].to_numpy(np.int32, (M, N)) == oracle.sptmm_i8_mt(Xs[i], pos, neg, 4)).all(), i
+    for o in ws + xb + cb:
+        o.free()
+    st.destroy()
+
+
 @pytest.mark.parametrize("kind", ["u16", "delta"])
 @pytest.mark.parametrize("dtype,act", [(np.float16, 1), (np.float32, 2)])
 def test_batched_launch_float_activations(kind, dtype, act):
