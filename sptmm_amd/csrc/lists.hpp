@@ -1116,9 +1116,11 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // A batched launch has workgroups enough to fill the chip along blockIdx.z, and every workgroup
     // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
     // per GEMV, four-row tiles 2.83 -> 2.76; nothing for the one-row u16 kernel, which waits on HBM only).
-    if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && MT == 1)) {
-        grid_x = (blocks + 1) / 2;
-        iters = 2;
+    // Eight-row tiles (110 KB at K=13824) take four: u16 lists 67 -> 70 %, gap streams level.
+    const int biters = MT == 8 ? 4 : 2;
+    if (a.batch >= 8 && iters == 1 && blocks >= biters && !(MODE == 0 && MT == 1)) {
+        grid_x = (blocks + biters - 1) / biters;
+        iters = biters;
     }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
                  a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale};
