@@ -385,7 +385,22 @@ static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
     wpb = wpb < 4 ? 4 : wpb > MAXW / per_cu ? MAXW / per_cu : wpb;
     if (tune_wpb > 0 && tune_wpb <= MAXW) wpb = tune_wpb;
     const int blocks = (a.tasks + wpb - 1) / wpb;
-    const int grid_x = blocks < cus * per_cu ? blocks : cus * per_cu;
+    int grid_x = blocks < cus * per_cu ? blocks : cus * per_cu;
+    // A batched launch fills the chip along blockIdx.z, and every workgroup pays 2.5 us per K-tile for staging before
+    // it walks (about 7 us per task): fewer workgroups with up to eight tasks per wavefront, as long as the launch's
+    // workgroups still come in full rounds over the compute units (config 4, M=16, 7 GEMVs per launch: 1 / 2 / 4 / 8
+    // tasks per wavefront 21.2 / 20.1 / 18.4 / 17.4 us per GEMV; 6 -- one and a fifth rounds -- 23.7 us).
+    if (a.batch >= 4 && blocks <= cus * per_cu) {
+        double best = 1e30;
+        int pick = 1;
+        for (int bi = 1; bi <= 8; bi *= 2) {
+            if (blocks < bi) break;
+            const long total = (long)a.batch * ((blocks + bi - 1) / bi), slots = (long)cus * per_cu;
+            const double cost = (double)((total + slots - 1) / slots) * (2.5 + 7.0 * bi);
+            if (cost < best - 1e-9) best = cost, pick = bi;
+        }
+        grid_x = (blocks + pick - 1) / pick;
+    }
     WideParams p{};
     p.w = (const uint8_t *)a.w, p.X = a.X, p.C = a.C;
     p.M = a.M, p.K = a.K, p.N = a.N, p.k_tile = h.k_tile, p.phases = h.phases, p.tasks = a.tasks, p.logL = ilog2(a.L);
