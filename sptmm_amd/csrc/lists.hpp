@@ -1116,11 +1116,23 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // A batched launch has workgroups enough to fill the chip along blockIdx.z, and every workgroup
     // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
     // per GEMV, four-row tiles 2.83 -> 2.76; nothing for the one-row u16 kernel, which waits on HBM only).
-    // Eight-row tiles (110 KB at K=13824) take four: u16 lists 67 -> 70 %, gap streams level.
-    const int biters = MT == 8 ? 4 : 2;
-    if (a.batch >= 8 && iters == 1 && blocks >= biters && !(MODE == 0 && MT == 1)) {
-        grid_x = (blocks + biters - 1) / biters;
-        iters = biters;
+    if (MT == 8 && a.batch >= 4 && wgs == 1) {
+        // Eight-row tiles (110 KB at K=13824: one workgroup per CU, ~2.5 us of staging against ~4 us per task): up to 16
+        // tasks per wavefront, as long as the launch's workgroups still come in full rounds over the compute units
+        // (K=13824 N=5120 split_k=64, 8 GEMVs per launch: 2 / 4 / 8 tasks per wavefront 17.6 / 15.9 / 15.2 us per GEMV,
+        // 12 -- one and a third rounds -- 18.9 us).
+        double best = 1e30;
+        int pick = iters;
+        for (int t = iters; t <= 16 && t <= blocks; t *= 2) {
+            const long total = (long)a.batch * ((blocks + t - 1) / t);
+            const double cost = (double)((total + slots - 1) / slots) * (2.5 + 4.0 * t);
+            if (cost < best - 1e-9) best = cost, pick = t;
+        }
+        grid_x = (blocks + pick - 1) / pick;
+        iters = (blocks + grid_x - 1) / grid_x;
+    } else if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && MT == 1)) {
+        grid_x = (blocks + 1) / 2;
+        iters = 2;
     }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
                  a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale};
