@@ -74,6 +74,7 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
     static constexpr int NW = MX ? MT / 4 : 1;              // dwords per gathered slot (int8)
     static constexpr int ND = MX ? MT / 4 : 1;              // result tiles
     v4i D[ND], Bp[ND], Bn[ND];                              // MX: 16x16 int32 result tiles and the +1 / -1 selectors
+    bool merged = false;                                    // MT = 8, columns of 32 or 64 lanes: one result tile sums lanes i, i+16 (, i+32, i+48)
     v4f Df;                                                 // MXF: the fp32 result tile ...
     v8h Bpf, Bnf;                                           // ... and its selectors
     A acc[MT];
@@ -87,11 +88,13 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
             return (A)(D[x][0] + D[x][1] + D[x][2] + D[x][3]);
     }
 
-    __device__ __forceinline__ void init()
+    // logL: log2 of the lanes that share a column (the matrix-unit sums of eight-row tiles depend on it)
+    __device__ __forceinline__ void init(int logL = 0)
     {
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[m] = (A)0;
         if constexpr (MX) {
+            merged = MT == 8 && logL >= 5;
             // Selector held by lane j + 16 g (k-block g, output column j): 1 where the byte of the A operand
             // at the same (g, byte) position is to be added into column j.  MT = 4: A = 4 entries x 4 rows,
             // column 4 g + row.  MT = 8: A = 2 entries x 8 rows, tile x takes k-blocks 2x and 2x + 1, column
@@ -104,7 +107,10 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                 if constexpr (MT == 4) {
                     e = o = (j >> 2) == g ? b : 0u;
                 } else {
-                    const bool on = (g >> 1) == x && (j >> 3) == (g & 1);
+                    // Two result tiles keep every lane's sums apart (tile x: k-blocks 2x, 2x+1 -> column 8 (g & 1) + row).
+                    // When lanes i and i+16 belong to one column anyway (32 lanes per column: k-blocks 0, 1 -> columns
+                    // 0..7, k-blocks 2, 3 -> 8..15; 64 lanes: all four -> 0..7) one tile does, with half the instructions.
+                    const bool on = merged ? (x == 0 && (j >> 3) == (logL == 5 ? g >> 1 : 0)) : ((g >> 1) == x && (j >> 3) == (g & 1));
                     e = on && !(j & 4) ? b : 0u;
                     o = on && (j & 4) ? b : 0u;
                 }
@@ -145,8 +151,10 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                 else
                     a = v4i{(int)r[e].v[0], (int)r[e].v[1], e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[0] : 0,
                             e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[1] : 0};
-#pragma unroll
-                for (int x = 0; x < ND; ++x) D[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[x] : Bp[x], D[x], 0, 0, 0);
+                D[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[0] : Bp[0], D[0], 0, 0, 0);
+                if constexpr (ND > 1) {
+                    if (!merged) D[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[1] : Bp[1], D[1], 0, 0, 0);  // (uniform)
+                }
             }
         } else if constexpr (MXF) {
 #pragma unroll
@@ -823,7 +831,7 @@ struct ListsBody {
                 store_lane_sums(p, pacc.acc, part, back, active, task, lane, wave, m0);
             } else {
             Sums<Act, MT> acc;
-            acc.init();
+            acc.init(p.logL);
 
             if constexpr (RF != 0) {
                 if (it > 0) {
@@ -938,6 +946,30 @@ struct ListsBody {
                 constexpr int ND = Sums<Act, MT>::ND;
                 const int logL = p.logL;
                 A t[ND];
+                bool merged_done = false;
+                if constexpr (Sums<Act, MT>::MX && MT == 8) {
+                    if (acc.merged) {
+                        // one tile: lane l, register r = rows i = 4 (l >> 4) + r, result column j = l & 15 holds activation
+                        // row j & 7 of the task's column j >> 3; the 16 i are the column's lanes i, i+16 (, i+32, i+48)
+                        A v = acc.tile_sum(0);
+                        v += swz16(v);
+                        v += __shfl_xor(v, 32, 64);
+                        const int m = lane & 7;
+                        if (p.W == 1) {
+                            if (active && lane < (logL == 5 ? 16 : 8) && m0 + m < p.M) {
+                                const int col = (task << (6 - logL)) + (lane >> 3);
+                                if constexpr (QUANT)
+                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)v * qinv[m] * p.w_scale;
+                                else
+                                    C[(size_t)(m0 + m) * p.N + col] = v;
+                            }
+                        } else if (lane < MT) {
+                            part[wave * MT + lane] = v;
+                        }
+                        merged_done = true;
+                    }
+                }
+                if (!merged_done) {
 #pragma unroll
                 for (int x = 0; x < ND; ++x) {
                     t[x] = acc.tile_sum(x);
@@ -979,6 +1011,7 @@ struct ListsBody {
                 } else if (lane < MT) {
                     part[wave * MT + lane] = t[0];
                 }
+                }  // two-tile epilogue
             } else {
                 store_lane_sums(p, acc.acc, part, back, active, task, lane, wave, m0);
             }
