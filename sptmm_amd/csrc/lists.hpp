@@ -1141,6 +1141,9 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // byte rows, batched: the tile is a quarter of the others' and the chip is filled along blockIdx.z; the largest
     // workgroup does best (headline shape, 32 GEMVs per launch: 5 wavefronts 77 %, 8 wavefronts 79 % of HBM peak)
     if (is_byte_rows<Act>() && a.batch) wpb = max_waves / a.W * a.W;
+    // eight-row tiles keep the matrix unit busy: a batched launch takes a wavefront count the four SIMDs share evenly
+    // (K=13824 N=5120, M=8, 10 -> 12 wavefronts: gap stream 48 -> 55 % of HBM peak, u16 lists level)
+    if (MT == 8 && a.batch >= 4 && a.W == 1 && wpb % 4 && (wpb + 3) / 4 * 4 <= max_waves) wpb = (wpb + 3) / 4 * 4;
     if (tune_wpb > 0 && tune_wpb <= max_waves && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;

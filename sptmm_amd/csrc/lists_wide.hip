@@ -383,6 +383,10 @@ static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
     const int per_cu = (size_t)a.lds_limit >= 2 * lds ? 2 : 1;  // workgroups whose tiles fit a compute unit together
     int wpb = (a.tasks + cus * per_cu - 1) / (cus * per_cu);
     wpb = wpb < 4 ? 4 : wpb > MAXW / per_cu ? MAXW / per_cu : wpb;
+    // The walk keeps the matrix unit busy (one instruction per entry), and a wavefront count that does not divide by
+    // the four SIMDs leaves some of them a third more work: batched launches, which are free to regroup their tasks,
+    // take a multiple of four (config 4, M=16, 10 -> 12 wavefronts: gap stream 17.9 -> 14.7 us per GEMV, u16 16.2 -> 16.0).
+    if (a.batch >= 4 && wpb % 4 && (wpb + 3) / 4 * 4 <= MAXW / per_cu) wpb = (wpb + 3) / 4 * 4;
     if (tune_wpb > 0 && tune_wpb <= MAXW) wpb = tune_wpb;
     const int blocks = (a.tasks + wpb - 1) / wpb;
     int grid_x = blocks < cus * per_cu ? blocks : cus * per_cu;
