@@ -1144,6 +1144,9 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // eight-row tiles keep the matrix unit busy: a batched launch takes a wavefront count the four SIMDs share evenly
     // (K=13824 N=5120, M=8, 10 -> 12 wavefronts: gap stream 48 -> 55 % of HBM peak, u16 lists level)
     if (MT == 8 && a.batch >= 4 && a.W == 1 && wpb % 4 && (wpb + 3) / 4 * 4 <= max_waves) wpb = (wpb + 3) / 4 * 4;
+    // four-row tiles on gap streams, batched, tile small enough for several workgroups per CU: eight wavefronts
+    // (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824 five do better)
+    if (MT == 4 && MODE != 0 && a.batch >= 4 && a.W == 1 && tile <= 40 * 1024 && max_waves >= 8) wpb = 8;
     if (tune_wpb > 0 && tune_wpb <= max_waves && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
