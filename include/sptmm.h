@@ -288,7 +288,9 @@ int sptmm_graph_destroy(void *graph);
  * stream between two events; 1 = stream synchronize after every launch, as the
  * reference does (main.cu:1456); 2 = one rotation captured into a HIP graph and
  * replayed; 3 = every rotation is ONE sptmm_gemv_i8_batched launch of all n_ws
- * GEMVs (C_dev must then hold n_ws * M * N outputs).  `stream` must come from sptmm_stream_create; the call returns after
+ * GEMVs (C_dev must then hold n_ws * M * N outputs); 4 = one GEMV per launch as in mode 0, launch i on the i % 4-th of
+ * four streams the call makes for itself (C_dev holds 4 * M * N outputs), timed from an event all four wait for to an
+ * event that waits for all four.  `stream` must come from sptmm_stream_create; the call returns after
  * the stream has drained.  Reports mean microseconds per launch, taken from two
  * events recorded on that stream. */
 int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X_dev, int M, void *C_dev,

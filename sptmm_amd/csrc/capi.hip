@@ -698,7 +698,8 @@ int measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *
                  void *stream, double *us_per_call)
 {
     if (!ws || n_ws < 1 || !X || !C || iters < 1 || !us_per_call) return fail(SPTMM_ERR_INVALID, "bad argument");
-    if (act < 0 || act > 4 || mode < 0 || mode > 3) return fail(SPTMM_ERR_INVALID, "bad act or mode");
+    if (act < 0 || act > 4 || mode < 0 || mode > 4) return fail(SPTMM_ERR_INVALID, "bad act or mode");
+    if (mode == 4 && act > ACT_F32) return fail(SPTMM_ERR_UNSUPPORTED, "timing over several streams takes int8, fp16 or fp32 activations");
     if (mode == 3 && act > ACT_F32) return fail(SPTMM_ERR_UNSUPPORTED, "batched timing takes int8, fp16 or fp32 activations");
     // act 3 / 4: the quantising GEMV on fp16 / bf16 rows (w_scale 1)
     auto launch = [&](const sptmm_weights *w) {
@@ -708,6 +709,9 @@ int measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *
     if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_measure_gemv needs a stream made by sptmm_stream_create");
     hipStream_t st = (hipStream_t)stream;
     hipEvent_t e0 = nullptr, e1 = nullptr;
+    constexpr int NSTREAMS = 4;
+    hipStream_t side[NSTREAMS] = {nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t side_done[NSTREAMS] = {nullptr, nullptr, nullptr, nullptr};
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     int rc = SPTMM_OK;
@@ -755,6 +759,28 @@ int measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *
         M_TRY(hipEventSynchronize(e1));
         M_TRY(hipEventElapsedTime(&ms, e0, e1));
         *us_per_call = (double)ms * 1000.0 / ((double)reps * n_ws);
+    } else if (mode == 4) {
+        // still one GEMV per launch, but launch i goes to stream i % 4 (default priority, like every stream here): independent
+        // GEMVs then overlap the ramp and the tail of their neighbours.  Outputs of the four streams side by side in C.
+        for (int s = 0; s < NSTREAMS; ++s) {
+            M_TRY(hipStreamCreateWithFlags(&side[s], hipStreamNonBlocking));
+            M_TRY(hipEventCreateWithFlags(&side_done[s], hipEventDisableTiming));
+        }
+        M_TRY(hipEventRecord(e0, st));
+        for (int s = 0; s < NSTREAMS; ++s) M_TRY(hipStreamWaitEvent(side[s], e0, 0));
+        for (int i = 0; i < iters; ++i) {
+            const int s = i % NSTREAMS;
+            rc = gemv_common(ws[i % n_ws], X, M, (int32_t *)C + (size_t)s * M * ws[0]->info.N, side[s], (ActType)act);
+            if (rc != SPTMM_OK) goto done;
+        }
+        for (int s = 0; s < NSTREAMS; ++s) {
+            M_TRY(hipEventRecord(side_done[s], side[s]));
+            M_TRY(hipStreamWaitEvent(st, side_done[s], 0));
+        }
+        M_TRY(hipEventRecord(e1, st));
+        M_TRY(hipEventSynchronize(e1));
+        M_TRY(hipEventElapsedTime(&ms, e0, e1));
+        *us_per_call = (double)ms * 1000.0 / iters;
     } else {
         M_TRY(hipEventRecord(e0, st));
         for (int i = 0; i < iters; ++i) {
@@ -773,6 +799,13 @@ done:
     if (graph) (void)hipGraphDestroy(graph);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
+    for (int s = 0; s < NSTREAMS; ++s) {
+        if (side[s]) {
+            (void)hipStreamSynchronize(side[s]);
+            (void)hipStreamDestroy(side[s]);
+        }
+        if (side_done[s]) (void)hipEventDestroy(side_done[s]);
+    }
     (void)hipStreamSynchronize(st);
     return rc;
 }

@@ -650,3 +650,33 @@ def test_threads_share_one_weights_object():
     for w in ws:
         w.free()
     assert not errors, errors
+
+
+@pytest.mark.parametrize("mode,outputs", [(0, 1), (1, 1), (2, 1), (3, 3), (4, 4)])
+def test_timing_entry_point_leaves_the_results_of_its_launches(mode, outputs):
+    """sptmm_measure_gemv issues the product's own launches: whatever the protocol (one stream, a host sync per launch,
+    a graph, batched, four streams), the output buffer afterwards holds the GEMV of the rows it was given."""
+    sp.device_init(0)
+    K, N, S, M = 2560, 640, 1536, 1
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    w = sp.Weights.upload_u16(pos, neg, K, 32)
+    ws = [w, w.clone(), w.clone()]
+    X = oracle.make_x_i8(41 + mode, M, K)
+    xb = sp.DeviceBuffer.from_numpy(X)
+    cb = sp.DeviceBuffer(4 * M * N * 4)
+    cb.fill(0xEE)
+    st = sp.Stream()
+    say("timing entry point, mode", mode)
+    us = sp.measure_gemv(ws, 0, xb, M, cb, 12, mode, st)
+    st.sync()
+    assert 0.0 < us < 1e5
+    got = cb.to_numpy(np.int32, (4, M * N))
+    want = oracle.sptmm_i8(X, pos, neg).reshape(-1)
+    for i in range(outputs):
+        assert (got[i] == want).all(), (mode, i)
+    with pytest.raises(sp.SptmmError):
+        sp.measure_gemv(ws, 0, xb, M, cb, 4, 5, st)
+    for o in (xb, cb):
+        o.free()
+    for o in ws:
+        o.free()
