@@ -1158,16 +1158,27 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // A batched launch has workgroups enough to fill the chip along blockIdx.z, and every workgroup
     // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
     // per GEMV, four-row tiles 2.83 -> 2.76; nothing for the one-row u16 kernel, which waits on HBM only).
-    if (MT == 8 && a.batch >= 4 && wgs == 1) {
-        // Eight-row tiles (110 KB at K=13824: one workgroup per CU, ~2.5 us of staging against ~4 us per task): up to 16
-        // tasks per wavefront, as long as the launch's workgroups still come in full rounds over the compute units
-        // (K=13824 N=5120 split_k=64, 8 GEMVs per launch: 2 / 4 / 8 tasks per wavefront 17.6 / 15.9 / 15.2 us per GEMV,
-        // 12 -- one and a third rounds -- 18.9 us).
+    if ((MT == 8 || (MT == 4 && MODE != 0)) && a.batch >= 4 && wgs == 1) {
+        // Multi-row tiles are expensive to stage (eight rows of K=13824: 110 KB, ~2.5 us against ~4 us per task) and their
+        // walks are bound by the LDS and the matrix unit rather than by HBM: up to 16 tasks per wavefront, chosen so that the
+        // launch's workgroups come in full rounds over the workgroups the chip holds at once (cost per round: staging
+        // + tasks per wavefront x one task's walk, in rough microseconds; only the ratio matters).  Measured, per GEMV:
+        // K=13824 N=5120 split_k=64, M=8, 8 u16 GEMVs per launch, 2 / 4 / 8 tasks per wavefront 17.6 / 15.9 / 15.2 us
+        // (12 tasks -- one and a third rounds -- 18.9 us); 14 gap-stream GEMVs, 8 / 12 tasks 10.1 / 9.8 us (10 tasks: 2.35
+        // rounds, 10.9 us); K=6912 N=2560 split_k=32, M=4, 32 gap-stream GEMVs, 2 / 5 / 10 tasks 2.18 / 2.01 / 1.94 us
+        // (int8 rows), 2.50 / 2.19 / 2.05 us (fp16 rows); K=13824, four fp16 rows, 2 / 12 tasks 16.1 / 11.6 us.
+        // u16 lists on four-row tiles wait on HBM and gain nothing from more than two tasks.
+        const size_t per_wg = tile + lists_behind_tile<Act, MT>(wpb);
+        const int by_lds = (int)((size_t)a.lds_limit / per_wg), by_regs = 4 * waves_per_simd / wpb;
+        const int resident = std::max(1, std::min(by_lds, by_regs));
+        const long at_once = (long)cus * resident;
+        const int row_tiles = (a.M + MT - 1) / MT;
+        const double stage = MT == 8 ? 2.5 : 2.0, walk = MT == 8 ? 4.0 : 5.7;
         double best = 1e30;
         int pick = iters;
-        for (int t = iters; t <= 16 && t <= blocks; t *= 2) {
-            const long total = (long)a.batch * ((blocks + t - 1) / t);
-            const double cost = (double)((total + slots - 1) / slots) * (2.5 + 4.0 * t);
+        for (int t = 1; t <= 16 && t <= blocks; ++t) {
+            const long total = (long)a.batch * row_tiles * ((blocks + t - 1) / t);
+            const double cost = (double)((total + at_once - 1) / at_once) * (stage + walk * t);
             if (cost < best - 1e-9) best = cost, pick = t;
         }
         grid_x = (blocks + pick - 1) / pick;
