@@ -387,18 +387,22 @@ static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
     // the four SIMDs leaves some of them a third more work: batched launches, which are free to regroup their tasks,
     // take a multiple of four (config 4, M=16, 10 -> 12 wavefronts: gap stream 17.9 -> 14.7 us per GEMV, u16 16.2 -> 16.0).
     if (a.batch >= 4 && wpb % 4 && (wpb + 3) / 4 * 4 <= MAXW / per_cu) wpb = (wpb + 3) / 4 * 4;
+    // ... and the largest workgroup does better still: fewer workgroups stage the tile (the activation rows come out of
+    // L2 once per workgroup and K-tile) and four wavefronts per SIMD hide more of the gathers' latency (same shape, 12 ->
+    // 16 wavefronts: u16 15.9 -> 15.4 us per GEMV, gap stream 14.2 -> 12.7 us; a lone u16 GEMV 27.9 -> 24.4 us HBM-cold
+    // on 160 of the 256 compute units, a lone gap-stream GEMV 23.8 -> 24.4 us, so that one keeps the smaller workgroups)
+    if ((a.batch >= 4 || MODE == 0) && wpb >= 8) wpb = MAXW / per_cu;  // (shapes with tasks enough to fill the chip that way)
     if (tune_wpb > 0 && tune_wpb <= MAXW) wpb = tune_wpb;
     const int blocks = (a.tasks + wpb - 1) / wpb;
     int grid_x = blocks < cus * per_cu ? blocks : cus * per_cu;
     // A batched launch fills the chip along blockIdx.z, and every workgroup pays 2.5 us per K-tile for staging before
-    // it walks (about 7 us per task): fewer workgroups with up to eight tasks per wavefront, as long as the launch's
+    // it walks (about 7 us per task): fewer workgroups with up to 16 tasks per wavefront, as long as the launch's
     // workgroups still come in full rounds over the compute units (config 4, M=16, 7 GEMVs per launch: 1 / 2 / 4 / 8
     // tasks per wavefront 21.2 / 20.1 / 18.4 / 17.4 us per GEMV; 6 -- one and a fifth rounds -- 23.7 us).
     if (a.batch >= 4 && blocks <= cus * per_cu) {
         double best = 1e30;
         int pick = 1;
-        for (int bi = 1; bi <= 8; bi *= 2) {
-            if (blocks < bi) break;
+        for (int bi = 1; bi <= 16 && bi <= blocks; ++bi) {
             const long total = (long)a.batch * ((blocks + bi - 1) / bi), slots = (long)cus * per_cu;
             const double cost = (double)((total + slots - 1) / slots) * (2.5 + 7.0 * bi);
             if (cost < best - 1e-9) best = cost, pick = bi;
