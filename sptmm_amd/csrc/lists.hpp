@@ -1143,7 +1143,9 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     if (is_byte_rows<Act>() && a.batch) wpb = max_waves / a.W * a.W;
     // eight-row tiles keep the matrix unit busy: a batched launch takes a wavefront count the four SIMDs share evenly
     // (K=13824 N=5120, M=8, 10 -> 12 wavefronts: gap stream 48 -> 55 % of HBM peak, u16 lists level)
-    if (MT == 8 && a.batch >= 4 && a.W == 1 && wpb % 4 && (wpb + 3) / 4 * 4 <= max_waves) wpb = (wpb + 3) / 4 * 4;
+    // -- and the largest workgroup does best: four wavefronts per SIMD, fewer workgroups staging (same shape, 12 -> 16
+    // wavefronts: gap stream 9.95 -> 9.46 us per GEMV, u16 lists 14.0 -> 13.8 us)
+    if (MT == 8 && a.batch >= 4 && a.W == 1 && max_waves >= 4) wpb = max_waves / 4 * 4;
     // four-row tiles on gap streams, batched, tile small enough for several workgroups per CU: eight wavefronts
     // (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824 five do better)
     if (MT == 4 && MODE != 0 && a.batch >= 4 && a.W == 1 && tile <= 40 * 1024 && max_waves >= 8) wpb = 8;
