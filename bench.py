@@ -35,6 +35,9 @@ TRAFFIC_SIDECAR = os.path.join(ROOT, "profiles", "traffic_lists_kernel_batched_i
 LAYER = [("q/o", 2560, 2560, 1536, 2), ("k/v", 2560, 640, 1536, 2), ("gate/up", 2560, 6912, 1536, 2),
          ("down", 6912, 2560, 4160, 1)]
 LARGE = ("large", 13824, 5120, 8320)  # config 4
+# nonzeros per column of the headline shape for the density leg: 3.7 % (the reference's default flags, -K 3072 -S 256,
+# are 8.3 %), 7.4, 12.5 (u16 lists as many bytes as i2s), 18.5, 25 % (8-bit gaps as many bytes as i2s)
+DENSITY_S = (256, 512, 864, 1280, 1728)
 
 
 def algorithmic_bytes(stream_bytes, m, k, n, act_bytes=1):
@@ -113,10 +116,11 @@ def main():
     ap.add_argument("--reps", type=int, default=0,
                     help="launches per timed loop of the legs (0: 1500, the headline shape's other encodings 4096); counter "
                          "runs under a profiler, where every launch is serialised, use a few dozen")
-    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,cfg4",
+    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,cfg4,density",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, sync-each-call, four streams), "
                          "others (delta and i2s encodings at the headline shape), cfg1 (the same matrix at M=4), cfg2 (gap "
                          "stream with fp16 rows), cfg3 (decoder-layer shapes, M=1 and 4), cfg4 (K=13824 N=5120, M=1/8/16), "
+                         "density (the headline shape at 3.7-25 % nonzeros against i2s), "
                          "copy (4 launches of a 1 GiB copy kernel, for counter calibration), ceiling (a pure streaming "
                          "read of as many bytes as one step moves); profiling runs use --legs none or one leg")
     a = ap.parse_args()
@@ -174,14 +178,17 @@ def main():
                 "batched_us": round(bat, 3), "batched_gbps": round(nb / bat / 1e3, 1), "batched_pct_roofline": pct(nb, bat),
                 "gemvs_per_batched_launch": len(groups[0])}
 
-    def run_matrix(label, k_rows, n_cols, s_nz, ms, lists=None, split=0):
+    def run_matrix(label, k_rows, n_cols, s_nz, ms, lists=None, split=0, from_dense=False):
         """The three encodings of one seeded matrix at the given row counts -> list of rows.  split = 0: the split
-        the library picks for the shape (sptmm_choose_split_k); the row's `split_k` says which."""
+        the library picks for the shape (sptmm_choose_split_k); the row's `split_k` says which.  from_dense: the gap
+        stream is built from the dense matrix (the builder for any ternary matrix), which walks gaps of more than 127
+        rows over zero slots of the tile instead of widening every gap to 16 bits."""
         Wm, p, n = lists if lists is not None else sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)
         rows = []
         # gap streams are packed for the number of activation rows they will meet: the GEMV stream (rows = 1) or the plain one
         makers = (("u16", lambda m: sp.Weights.upload_u16(p, n, k_rows, split)),
-                  ("delta", lambda m: sp.Weights.upload_delta(p, n, k_rows, split, rows=m)),
+                  ("delta", (lambda m: sp.Weights.upload_dense(Wm, sp.KIND_DELTA, split, rows=m)) if from_dense else
+                            (lambda m: sp.Weights.upload_delta(p, n, k_rows, split, rows=m))),
                   ("i2s", lambda m: sp.Weights.upload_i2s(Wm)))
         refs = {}
         for enc, mk in makers:
@@ -197,7 +204,8 @@ def main():
                     refs[m] = got
                     checks.append(("%s M=%d" % (label, m), Xm, p, n, got, s_nz))
                 r = {"shape": label, "K": k_rows, "N": n_cols, "S": s_nz, "M": m, "enc": enc, "split_k": w.info["split_k"],
-                     "row_bytes": w.info["row_bytes"], "bit_exact_across_encodings": bool((got == refs[m]).all())}
+                     "row_bytes": w.info["row_bytes"], "delta_bits": w.info["delta_bits"], "zero_slot_detours": w.info["stones"],
+                     "bit_exact_across_encodings": bool((got == refs[m]).all())}
                 r.update(time_encoding(w, 0, Xm, m, n_cols, k_rows))
                 rows.append(r)
             w.free()
@@ -323,6 +331,25 @@ def main():
             ww.free()
         configs["cfg4_large"] = rows
 
+    density = None
+    if "density" in legs:
+        # Where index lists overtake the 2-bit baseline: the same shape at fewer nonzeros per column.  i2s stores
+        # every weight (K*N/4 bytes whatever S), the lists 2 bytes per nonzero, gap streams 1 byte per nonzero plus one
+        # per zero slot visited on the way over a gap of more than 127 rows.
+        rows = []
+        for s_nz in DENSITY_S:
+            rows += run_matrix("density %.1f %%" % (100.0 * s_nz / K), K, N, s_nz, (1,), from_dense=True)
+        cross = []
+        for s_nz in DENSITY_S:
+            mine = [r for r in rows if r["S"] == s_nz]
+            i2s_us = next(r["batched_us"] for r in mine if r["enc"] == "i2s")
+            best = min((r for r in mine if r["enc"] != "i2s"), key=lambda r: r["batched_us"])
+            cross.append({"S": s_nz, "density_pct": round(100.0 * s_nz / K, 1), "best_lists_enc": best["enc"],
+                          "lists_batched_us": best["batched_us"], "i2s_batched_us": i2s_us,
+                          "lists_over_i2s": round(best["batched_us"] / i2s_us, 3)})
+        wins = [c["density_pct"] for c in cross if c["lists_over_i2s"] < 1.0]
+        density = {"shapes": rows, "against_i2s": cross, "lists_beat_i2s_up_to_density_pct": max(wins) if wins else None}
+
     gbps = nbytes / us_gemv / 1e3
     traffic, traffic_src = None, None
     if os.path.exists(TRAFFIC_SIDECAR):
@@ -353,8 +380,10 @@ def main():
             "hbm_70pct_one_gemv_per_launch_over_four_streams": (single["cold_four_streams_pct_roofline"] >= 70.0) if single else None,
             "beats_i2s_at_m1_batched": (us_gemv < i2s_m1["batched_us"]) if i2s_m1 else None,
             "beats_i2s_at_m1_one_per_launch": (single["cold_us"] < i2s_m1["alone_cold_us"]) if i2s_m1 and single else None,
+            # at BASELINE's 59 % nonzeros the lists hold 4.7x (gap stream 2.4x) the bytes of i2s; they win where they are smaller
+            "beats_i2s_batched_up_to_density_pct": density["lists_beat_i2s_up_to_density_pct"] if density else None,
         },
-        "single_launch": single, "other_encodings": others, "configs": configs,
+        "single_launch": single, "other_encodings": others, "configs": configs, "density_sweep": density,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_src,

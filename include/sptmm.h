@@ -62,6 +62,9 @@ typedef struct sptmm_winfo {
     int k_tile;      /* wide streams: rows per K-tile (0 for every other stream) */
     int row_bytes;   /* 8-bit gap streams: bytes per row of the activation tile the visiting order was scheduled for,
                       * 1 (sptmm_*_rows with rows = 1) or 4; 0 for every other stream */
+    int stones;      /* 1: 8-bit gap stream of a matrix too sparse for byte gaps throughout -- the activation tile keeps 16 zero
+                      * slots behind every 112 rows, the stream holds tile positions, and a gap of more than 127 positions
+                      * is walked over zero slots (entries that add nothing); 0 for every other stream */
 } sptmm_winfo;
 
 typedef struct sptmm_weights sptmm_weights; /* opaque; owns its device buffer */

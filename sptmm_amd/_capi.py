@@ -54,7 +54,7 @@ class DevInfo(C.Structure):
 class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
                 ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64),
-                ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int), ("row_bytes", C.c_int)]
+                ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int), ("row_bytes", C.c_int), ("stones", C.c_int)]
 
 
 def lib_path() -> str:

@@ -24,6 +24,7 @@ struct sptmm_weights {
     int n_min = 0, n_max = 0;
     int index_shift = 0;  // u16 streams: fields are row << index_shift
     bool byte_rows = false;  // 8-bit gap stream scheduled for a tile of one byte per row
+    bool stones = false;     // 8-bit gap stream of tile positions (zero slots behind every 112 rows of the tile)
     bool wide = false;    // wide stream (K-tiled, 16-byte slots): `wh` describes it
     WideHeader wh;
 };
@@ -142,6 +143,7 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.n_max = w->n_max;
     a.index_shift = w->index_shift;
     a.byte_rows = w->byte_rows;
+    a.stones = w->stones;
     a.ragged = w->info.ragged;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
@@ -229,6 +231,30 @@ int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, in
         if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
         int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
         if (bits < 0) return bits;
+        if (bits == 16 && K + 64 <= 65535) {
+            // Some gap is too long for a byte (the reference narrows every gap to u8 unchecked, main.cu:376-394).  The
+            // builder for arbitrary matrices can walk long gaps over zero slots of the tile; take its stream where
+            // that is smaller than 16-bit gaps throughout.
+            std::vector<int8_t> W((size_t)K * N, 0);
+            for (int sign = 0; sign < 2; ++sign) {
+                const uint16_t *l = sign ? neg : pos;
+                for (int c = 0; c < N; ++c)
+                    for (int i = 0; i < S / 2; ++i) {
+                        const uint16_t r = l[(size_t)c * (S / 2) + i];
+                        if (r >= K) return fail(SPTMM_ERR_INVALID, "row index %d out of range in column %d", (int)r, c);
+                        W[(size_t)c * K + r] = sign ? (int8_t)-1 : (int8_t)1;
+                    }
+            }
+            sptmm_weights *alt = nullptr;
+            if (sptmm_weights_upload_dense_rows(W.data(), K, N, SPTMM_KIND_DELTA, split_k, rows, &alt) == SPTMM_OK) {
+                if (alt->info.delta_bits == 8) {
+                    alt->info.S = S;
+                    *out = alt;
+                    return SPTMM_OK;
+                }
+                sptmm_weights_free(alt);
+            }
+        }
         std::vector<uint8_t> host(sptmm_pack_delta_bytes(N, S, split_k, bits));
         if (int rc = sptmm_pack_delta_rows(pos, neg, K, N, S, split_k, bits, rows, host.data())) return rc;
         sptmm_weights *w = new (std::nothrow) sptmm_weights();
@@ -290,6 +316,8 @@ int sptmm_weights_upload_dense_rows(const int8_t *W, int K, int N, int kind, int
         w->index_shift = kind == SPTMM_KIND_U16 ? ragged_index_shift(K) : 0;
         w->byte_rows = kind == SPTMM_KIND_DELTA && bits == 8 && rows == 1;
         w->info.row_bytes = kind == SPTMM_KIND_DELTA && bits == 8 ? (rows == 1 ? 1 : 4) : 0;
+        w->stones = kind == SPTMM_KIND_DELTA && bits == 8 && *(const uint32_t *)host.data() == RAGGED_MAGIC_STONES;
+        w->info.stones = w->stones ? 1 : 0;
         return finish_upload(w, host, out);
     });
 }
@@ -489,7 +517,8 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
             // the per-task counts are what the kernel trusts most: keep them inside [n_min, n_max]
             const uint32_t *pre = (const uint32_t *)host.data();
             const uint16_t *counts = (const uint16_t *)(host.data() + 16);
-            bool ok = pre[0] == RAGGED_MAGIC && pre[1] == (uint32_t)h.tasks && pre[2] == (uint32_t)h.n_max && pre[3] == (uint32_t)h.n_min;
+            const bool stones = h.kind == SPTMM_KIND_DELTA && h.delta_bits == 8 && pre[0] == RAGGED_MAGIC_STONES && stone_tile_rows(h.K) + 64 <= 65535;
+            bool ok = (pre[0] == RAGGED_MAGIC || stones) && pre[1] == (uint32_t)h.tasks && pre[2] == (uint32_t)h.n_max && pre[3] == (uint32_t)h.n_min;
             for (int t = 0; ok && t < h.tasks; ++t) ok = counts[t] >= h.n_min && counts[t] <= h.n_max;
             if (!ok) return fail(SPTMM_ERR_INVALID, "%s: corrupt count table", path);
         }
@@ -504,6 +533,8 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         w->index_shift = h.kind == SPTMM_KIND_DELTA ? 0 : h.index_shift;
         w->byte_rows = h.kind == SPTMM_KIND_DELTA && h.index_shift == 2;
         w->info.row_bytes = h.kind == SPTMM_KIND_DELTA && h.delta_bits == 8 ? (w->byte_rows ? 1 : 4) : 0;
+        w->stones = h.ragged && h.kind == SPTMM_KIND_DELTA && h.delta_bits == 8 && *(const uint32_t *)host.data() == RAGGED_MAGIC_STONES;
+        w->info.stones = w->stones ? 1 : 0;
         return finish_upload(w, host, out);
     });
 }
@@ -526,7 +557,7 @@ int sptmm_gemv_batched(const sptmm_weights *const *ws, const void *const *X, voi
             if (!ws[i] || !X[i] || !C[i]) return fail(SPTMM_ERR_INVALID, "null pointer in batch entry %d", i);
             const sptmm_winfo &a = ws[0]->info, &b = ws[i]->info;
             if (a.kind != b.kind || a.K != b.K || a.N != b.N || a.S != b.S || a.split_k != b.split_k || a.delta_bits != b.delta_bits ||
-                a.ragged != b.ragged || a.k_tile != b.k_tile || a.row_bytes != b.row_bytes || ws[0]->wide != ws[i]->wide ||
+                a.ragged != b.ragged || a.k_tile != b.k_tile || a.row_bytes != b.row_bytes || a.stones != b.stones || ws[0]->wide != ws[i]->wide ||
                 (ws[0]->wide && memcmp(&ws[0]->wh, &ws[i]->wh, sizeof(WideHeader)) != 0) || ws[0]->task_stride != ws[i]->task_stride ||
                 ws[0]->n_min != ws[i]->n_min)
                 return fail(SPTMM_ERR_INVALID, "batch entry %d differs in kind or shape from entry 0", i);

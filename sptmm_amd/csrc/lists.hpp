@@ -475,7 +475,11 @@ struct ListParams {
     int iters;  // tasks each wavefront walks: ceil(tasks / (gridDim.x * waves))
     int quant;      // quantising kernels: X holds 1 = fp16, 2 = bf16 values
     float w_scale;  // quantising kernels: factor applied to every output
+    int stones;     // 8-bit gap streams of tile positions: the tile keeps 16 zero slots behind every 112 rows
 };
+
+// rows of the activation tile in front of its 64 trailing zero rows
+static inline int lists_tile_rows(const GemvArgs &a) { return a.stones ? stone_tile_rows(a.K) : a.K; }
 
 constexpr int LISTS_MAX_WAVES = 8;  // 512 threads: two wavefronts per SIMD, 256 VGPRs each
 // Multi-row int8 tiles do several times the arithmetic per stream byte, and a large K leaves
@@ -655,7 +659,10 @@ struct ListsBody {
     {
         constexpr int NR = RF > 0 ? RF : 0;               // full rounds of the straight-line body (RF == -1: none, tails only)
         constexpr int NB = RF > 0 ? RF : RF == 0 ? RING : 1;
-        A *part = reinterpret_cast<A *>(smem + (size_t)(p.K + ZROWS) * SLOT);
+        // stepping-stone streams: item i (16 rows) goes to item i + i/7 of the tile, every eighth item stays zero
+        const int tile_rows = p.stones ? STONE_BLOCK * ((p.K + STONE_ROWS - 1) / STONE_ROWS) : p.K;
+        auto place = [&](int item) { return p.stones ? item + item / (STONE_ROWS / 16) : item; };
+        A *part = reinterpret_cast<A *>(smem + (size_t)(tile_rows + ZROWS) * SLOT);
         const int tid = threadIdx.x, nt = blockDim.x;
         const int lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
         const int m0 = blockIdx.y * MT;
@@ -743,18 +750,18 @@ struct ListsBody {
             for (int i = 0; i < Q::HOLD; ++i)
                 if (tid + i * nt < items) {
                     Q::quantise(xq[i], p.quant, sc, xr[0]);
-                    St::store(smem, tid + i * nt, xr[0]);
+                    St::store(smem, place(tid + i * nt), xr[0]);
                 }
             for (int item = tid + Q::HOLD * nt; item < items; item += nt) {
                 uint4 r[2 * MT];
                 Q::load(Xq, p.M, p.K, m0, item, r);
                 Q::quantise(r, p.quant, sc, xr[0]);
-                St::store(smem, item, xr[0]);
+                St::store(smem, place(item), xr[0]);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < St::XI; ++i)
-                if (tid + i * nt < items) St::store(smem, tid + i * nt, xr[i]);
+                if (tid + i * nt < items) St::store(smem, place(tid + i * nt), xr[i]);
             if constexpr (TWIN) {
 #pragma unroll
                 for (int i = 0; i < St::XI; ++i)
@@ -777,7 +784,7 @@ struct ListsBody {
             for (int item = tid + St::XI * nt; item < items; item += nt) {
                 uint4 r[St::NLOAD];
                 St::load(X, p.M, p.K, m0, item, r);
-                St::store(smem, item, r);
+                St::store(smem, place(item), r);
                 if constexpr (TWIN) {
 #pragma unroll
                     for (int j = 0; j < St::NLOAD; ++j) xmax = pk_absmax16(xmax, r[j]);
@@ -786,7 +793,15 @@ struct ListsBody {
         }
         // rows K.. read as zero
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
-            reinterpret_cast<u32 *>(smem + (size_t)p.K * SLOT)[i] = 0u;
+            reinterpret_cast<u32 *>(smem + (size_t)tile_rows * SLOT)[i] = 0u;
+        if (p.stones) {
+            // the zero slots inside the tile: every eighth item, and what the last block holds beyond row K-1
+            constexpr int DW = 4 * SLOT;  // dwords per item
+            for (int i = tid; i < tile_rows / 16 * DW; i += nt) {
+                const int j = i / DW;
+                if (j % 8 == 7 || j - j / 8 >= items) reinterpret_cast<u32 *>(smem)[i] = 0u;
+            }
+        }
         // TWIN: one flag per wavefront behind the per-wavefront sums, folded by every thread after the barrier
         u32 *nf_flags = reinterpret_cast<u32 *>(part + waves * MT);
         if constexpr (TWIN) {
@@ -1102,7 +1117,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     static const int tune_wpb = getenv("SPTMM_WAVES_PER_WG") ? atoi(getenv("SPTMM_WAVES_PER_WG")) : 0;
     static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
     constexpr int SLOT = slot_bytes<Act, MT>();
-    const size_t tile = (size_t)(a.K + 64) * SLOT;
+    const size_t tile = (size_t)(lists_tile_rows(a) + 64) * SLOT;
     // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better
     const bool roomy = a.batch && 2 * (tile + lists_behind_tile<Act, MT>(LISTS_MAX_WAVES)) <= (size_t)a.lds_limit;
     const int max_waves = a.quant || roomy ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>();
@@ -1190,8 +1205,8 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         iters = 2;
     }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
-                 a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale};
-    size_t lds = (size_t)(a.K + 64) * SLOT + lists_behind_tile<Act, MT>(wpb);
+                 a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale, a.stones};
+    size_t lds = tile + lists_behind_tile<Act, MT>(wpb);
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     if (a.batch) {
@@ -1219,7 +1234,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         if constexpr (sizeof(Act) == 1) {
             auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, true>;
             // + room for the per-wavefront sums of a full workgroup, the row maxima and the rows' 1/s
-            lds = (size_t)(a.K + 64) * SLOT + (size_t)(2 * LISTS_MAX_WAVES + 1) * MT * 4;
+            lds = tile + (size_t)(2 * LISTS_MAX_WAVES + 1) * MT * 4;
             if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
             static std::atomic<size_t> lds_granted_q{48 * 1024};
             if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_q)) return rc;
@@ -1281,7 +1296,7 @@ static int launch_lists_m(const GemvArgs &a, hipStream_t st)
     // per-wavefront sums, and for quantising launches the row maxima and scales as well
     auto fits = [&](size_t slot, int mt, size_t behind) {
         const size_t extra = a.quant ? (size_t)(2 * LISTS_MAX_WAVES + 1) * mt * 4 : behind;
-        return (size_t)(a.K + 64) * slot + extra <= (size_t)a.lds_limit;
+        return (size_t)(lists_tile_rows(a) + 64) * slot + extra <= (size_t)a.lds_limit;
     };
     if constexpr (sizeof(Act) == 1) {
         if (a.M >= 5 && fits(slot_bytes<Act, 8>(), 8, lists_behind_tile<Act, 8>(lists_max_waves<Act, 8, false>())))

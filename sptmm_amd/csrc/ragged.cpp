@@ -28,6 +28,7 @@ struct RaggedPlan {
     Geometry g;
     int K = 0, kind = 0, bits = 0, esz = 2, hdr = 0, shift = 0;
     int bank_shift = 0;  // 8-bit gap streams: LDS bank = (row >> bank_shift) mod 32 (2: tiles of one byte per row)
+    bool stones = false; // 8-bit gap stream of tile positions, long gaps walked over the tile's zero slots
     std::vector<std::vector<uint16_t>> rows[2];  // [sign][column]: ascending row lists
     std::vector<int> n_task;
     int n_min = 0, n_max = 0;
@@ -36,6 +37,36 @@ struct RaggedPlan {
 };
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// The zero slot a walk at position `cur` steps to next on its way up: the farthest one within 127 positions.
+int stone_ahead(int cur)
+{
+    const int t = cur + 127;
+    return t % STONE_BLOCK >= STONE_ROWS ? t : STONE_BLOCK * (t / STONE_BLOCK) - 1;
+}
+
+// Stepping-stone stream: the positions the 64 lanes of one sign of a task visit, in ascending order and without padding.
+// Lane v of a column owns entries [v*n0, (v+1)*n0) of the column's sorted list (n0 = the task's longest list divided over
+// its lanes); wherever two of them lie more than 127 positions apart, zero slots are put between them.  -> longest run
+int stone_runs(const RaggedPlan &pl, int task, int sign, int n0, std::vector<uint16_t> (&run)[64])
+{
+    const Geometry &g = pl.g;
+    size_t longest = 0;
+    for (int lane = 0; lane < 64; ++lane) {
+        const std::vector<uint16_t> &e = pl.rows[sign][task * g.G + lane / g.L];
+        const int cnt = (int)e.size(), first = (lane % g.L) * n0;
+        std::vector<uint16_t> &r = run[lane];
+        r.clear();
+        for (int i = first; i < first + n0 && i < cnt; ++i) {
+            const int p = stone_pos(e[i]);
+            if (!r.empty())
+                while (p - (int)r.back() > 127) r.push_back((uint16_t)stone_ahead(r.back()));
+            r.push_back((uint16_t)p);
+        }
+        longest = std::max(longest, r.size());
+    }
+    return (int)longest;
+}
 
 // u16 stream, 64 lanes per column: the column's entries, ordered by bank, are dealt round-robin
 // over its nd half-wavefronts; half-wavefront d gets this many of cnt
@@ -115,11 +146,33 @@ int ragged_plan(const int8_t *W, int K, int N, int kind, int split_k, int bits_r
                     if (i % n && e[i] - e[i - 1] > 127) fits8 = false;
                 if (cnt % n && K - e[cnt - 1] > 127) fits8 = false;
             }
-        if (bits_req == 8 && !fits8) return fail(SPTMM_ERR_UNSUPPORTED, "a gap does not fit 8 bits (signed)");
-        pl->bits = bits_req ? bits_req : (fits8 ? 8 : 16);
-        pl->esz = pl->bits / 8;
         pl->hdr = 256;
         pl->shift = 0;
+        pl->bits = bits_req ? bits_req : (fits8 ? 8 : 16);
+        if (!fits8 && bits_req != 16) {
+            // Some gap is too long for a signed byte: walk it over zero slots of the tile (the task grows by the longest
+            // detour of its lanes) where that takes fewer bytes than 16-bit gaps, or where 8 bits were asked for.
+            if (stone_tile_rows(K) + 64 > 65535) {
+                if (bits_req == 8) return fail(SPTMM_ERR_UNSUPPORTED, "a gap does not fit 8 bits (signed), and K is too large for a tile with zero slots");
+            } else {
+                std::vector<int> with_stones(g.tasks, 1);
+                if (g.W > 1) return fail(SPTMM_ERR_UNSUPPORTED, "gap streams take at most 64 lanes per column");
+                parallel_for(g.tasks, [&](int t) {
+                    std::vector<uint16_t> run[64];
+                    for (int sign = 0; sign < 2; ++sign) with_stones[t] = std::max(with_stones[t], stone_runs(*pl, t, sign, pl->n_task[t], run));
+                });
+                size_t bytes8 = 0, bytes16 = 0;
+                for (int t = 0; t < g.tasks; ++t) bytes8 += 256 + (size_t)128 * with_stones[t], bytes16 += 256 + (size_t)256 * pl->n_task[t];
+                if (bits_req == 8 || bytes8 < bytes16) {
+                    pl->stones = true;
+                    pl->bits = 8;
+                    pl->n_task = with_stones;
+                    pl->n_max = *std::max_element(pl->n_task.begin(), pl->n_task.end());
+                    pl->n_min = *std::min_element(pl->n_task.begin(), pl->n_task.end());
+                }
+            }
+        }
+        pl->esz = pl->bits / 8;
     }
     pl->stride = pl->hdr + (size_t)128 * pl->esz * pl->n_max;
     if (pl->n_max > 65535) return fail(SPTMM_ERR_UNSUPPORTED, "more than 65535 entries per lane");
@@ -132,7 +185,7 @@ int ragged_plan(const int8_t *W, int K, int N, int kind, int split_k, int bits_r
 void put_counts(const RaggedPlan &pl, uint8_t *base)
 {
     uint32_t *pre = (uint32_t *)base;
-    pre[0] = RAGGED_MAGIC;
+    pre[0] = pl.stones ? RAGGED_MAGIC_STONES : RAGGED_MAGIC;
     pre[1] = (uint32_t)pl.g.tasks;
     pre[2] = (uint32_t)pl.n_max;
     pre[3] = (uint32_t)pl.n_min;
@@ -205,6 +258,22 @@ void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
         const int n = pl.n_task[task];
         uint8_t *t = base + (size_t)task * pl.stride;
         std::vector<uint16_t> rows[2][64];
+        if (pl.stones) {
+            // runs of positions; a lane that is done (or owns nothing) steps to the zero slots behind its block and stays
+            int n0 = 1;
+            for (int sign = 0; sign < 2; ++sign)
+                for (int cc = 0; cc < g.G; ++cc) n0 = std::max(n0, ceil_div((int)pl.rows[sign][task * g.G + cc].size(), g.L));
+            for (int sign = 0; sign < 2; ++sign) {
+                stone_runs(pl, task, sign, n0, rows[sign]);
+                for (int lane = 0; lane < 64; ++lane) {
+                    std::vector<uint16_t> &r = rows[sign][lane];
+                    const int rest = r.empty() ? STONE_ROWS : STONE_BLOCK * (r.back() / STONE_BLOCK) + STONE_ROWS;
+                    r.resize(n, (uint16_t)rest);
+                }
+            }
+            write_task_runs8(t, n, 65535, rows, pl.bank_shift);
+            return;
+        }
         for (int sign = 0; sign < 2; ++sign)
             for (int lane = 0; lane < 64; ++lane) {
                 const std::vector<uint16_t> &e = pl.rows[sign][task * g.G + lane / g.L];
@@ -327,8 +396,10 @@ int sptmm_unpack_ragged(const void *packed, int K, int N, int kind, int split_k,
         const int esz = gaps ? bits / 8 : 2, hdr = gaps ? 256 : 0, sh = gaps ? 0 : ragged_index_shift(K);
         const uint32_t *pre = (const uint32_t *)packed;
         const uint32_t n_max = pre[2];
-        if (pre[0] != RAGGED_MAGIC || pre[1] != (uint32_t)g.tasks || n_max < 1 || n_max > 65535 || pre[3] < 1 || pre[3] > n_max)
+        const bool stones = gaps && bits == 8 && pre[0] == RAGGED_MAGIC_STONES;
+        if ((pre[0] != RAGGED_MAGIC && !stones) || pre[1] != (uint32_t)g.tasks || n_max < 1 || n_max > 65535 || pre[3] < 1 || pre[3] > n_max)
             return fail(SPTMM_ERR_INVALID, "not a ragged stream of this shape");
+        const int tile_rows = stones ? stone_tile_rows(K) : K;
         const uint16_t *counts = (const uint16_t *)((const uint8_t *)packed + 16);
         const uint8_t *base = (const uint8_t *)packed + ragged_counts_bytes(g.tasks);
         const size_t stride = hdr + (size_t)128 * esz * n_max;
@@ -351,12 +422,13 @@ int sptmm_unpack_ragged(const void *packed, int K, int N, int kind, int split_k,
                             const uint8_t *cell = t + hdr + slot_offset((int)n, esz, sign, lane, i);
                             const int f = esz == 1 ? (gaps ? (int)(int8_t)*cell : (int)*cell) : (int)*(const uint16_t *)cell;
                             row = gaps ? row + f : f >> sh;
-                            if (row < 0 || row >= K + 64) {
+                            if (row < 0 || row >= tile_rows + 64) {
                                 bad[task] = 1;
                                 continue;
                             }
-                            if (row >= K) continue;  // padding
-                            int8_t &w = W[(size_t)col * K + row];
+                            const int r = stones ? (row < tile_rows ? stone_row(row) : K) : row;
+                            if (r < 0 || r >= K) continue;  // padding, or a zero slot on the way over a long gap
+                            int8_t &w = W[(size_t)col * K + r];
                             if (w) bad[task] = 1;  // a row may appear once per column
                             w = sign ? (int8_t)-1 : (int8_t)1;
                         }

@@ -183,17 +183,80 @@ def test_gap_stream_for_single_rows_holds_the_same_matrix_on_other_banks(split):
     assert res[1, 0] > res[1, 2] + 0.5 and res[0, 2] > res[0, 0] + 0.5, res  # and clearly worse on the other tile
 
 
-def test_sparse_matrix_takes_16_bit_gaps_and_8_bit_request_fails():
+def stone_pos(r):
+    """Position of row r in a tile that keeps 16 zero slots behind every 112 rows."""
+    return r + 16 * (r // 112)
+
+
+def walks_of(packed, n_max, table, task, sign):
+    """-> [64][n] positions the lanes of one sign of a gap-stream task visit, and n."""
+    stride = 256 + 128 * n_max
+    t = packed[table + task * stride:table + (task + 1) * stride]
+    n = int(packed[16 + 2 * task:][:2].view(np.uint16)[0])
+    out = np.empty((64, n), int)
+    for lane in range(64):
+        first = int(t[sign * 128 + 2 * lane: sign * 128 + 2 * lane + 2].view(np.uint16)[0])
+        gaps = t[[256 + slot_offset(n, 1, sign, lane, j) for j in range(n)]].view(np.int8).astype(int)
+        assert gaps[0] == 0
+        out[lane] = first + np.cumsum(gaps)
+    return out, n
+
+
+@pytest.mark.parametrize("K,N,split,p", [(6912, 32, 32, 0.01), (6912, 32, 16, 0.04), (2560, 64, 8, 0.02), (3072, 48, 16, 0.04), (2560, 16, 64, 0.02)])
+def test_sparse_matrix_walks_long_gaps_over_zero_slots(K, N, split, p):
+    """Gaps of more than 127 rows: an 8-bit stream of tile positions (16 zero slots behind every 112 rows) whose lanes
+    step over zero slots.  Every lane visits exactly the positions of its share of the sorted list, plus zero slots
+    only; every step fits a signed byte; what unpacks is the matrix."""
+    W = sp.generate_ternary_iid(K, N, 5, p, p)
+    W[0] = 0          # an empty column
+    W[1] = 0
+    W[1, K - 1] = 1   # one entry at the far end
+    packed, inf = sp.pack_ragged(W, DELTA, split, bits=8)
+    assert inf["bits"] == 8 and packed[:4].tobytes() == b"SPTS"
+    assert (sp.unpack_ragged(packed, K, N, DELTA, split, 8) == W).all()
+    G, L = 64 // split, split
+    tasks = N // G
+    table = -(-(16 + 2 * tasks) // 256) * 256
+    tile = 128 * -(-K // 112)
+    grew = 0
+    for task in range(tasks):
+        n0 = max(1, max(-(-int((W[task * G + c] == v).sum()) // L) for c in range(G) for v in (1, -1)))
+        for sign, val in ((0, 1), (1, -1)):
+            walks, n = walks_of(packed, inf["n_max"], table, task, sign)
+            grew += n - n0
+            assert n >= n0 and walks.min() >= 0 and walks.max() < tile
+            assert np.abs(np.diff(walks, axis=1)).max(initial=0) <= 128 and np.diff(walks, axis=1).max(initial=0) <= 127
+            for lane in range(64):
+                rows = np.flatnonzero(W[task * G + lane // L] == val)
+                mine = [stone_pos(int(r)) for r in rows[(lane % L) * n0:(lane % L + 1) * n0]]
+                seen = walks[lane]
+                real = sorted(int(x) for x in seen if x % 128 < 112)
+                assert real == mine, (task, sign, lane)   # every other visit is a zero slot
+    assert grew > 0  # some task did need a detour
+    # the same stream for tiles of one byte per row: same size, same matrix
+    p1, i1 = sp.pack_ragged(W, DELTA, split, bits=8, rows=1)
+    assert i1 == inf and len(p1) == len(packed) and (sp.unpack_ragged(p1, K, N, DELTA, split, 8) == W).all()
+
+
+def test_gap_width_is_chosen_by_size():
+    """bits = 0: byte gaps where every gap fits; else the smaller of the stream with zero-slot detours and 16-bit gaps."""
     K, N = 6912, 32
-    W = sp.generate_ternary_iid(K, N, 5, 0.01, 0.01)
-    packed, inf = sp.pack_ragged(W, DELTA, 32)
-    assert inf["bits"] == 16
-    assert (sp.unpack_ragged(packed, K, N, DELTA, 32, 16) == W).all()
-    with pytest.raises(sp.SptmmError):
-        sp.pack_ragged(W, DELTA, 32, bits=8)
     dense = sp.generate_ternary_iid(K, N, 5, 0.3, 0.3)
+    packed, inf = sp.pack_ragged(dense, DELTA, 32)
+    assert inf["bits"] == 8 and packed[:4].tobytes() == b"SPTR"
     p16, i16 = sp.pack_ragged(dense, DELTA, 32, bits=16)  # the wide form may always be asked for
     assert i16["bits"] == 16 and (sp.unpack_ragged(p16, K, N, DELTA, 32, 16) == dense).all()
+    for p in (0.002, 0.01, 0.03, 0.06):
+        W = sp.generate_ternary_iid(K, N, 7, p, p)
+        auto, ia = sp.pack_ragged(W, DELTA, 16)
+        p8, i8 = sp.pack_ragged(W, DELTA, 16, bits=8)
+        p16, i16 = sp.pack_ragged(W, DELTA, 16, bits=16)
+        assert i8["bits"] == 8 and i16["bits"] == 16 and p16[:4].tobytes() == b"SPTR"
+        assert len(auto) == min(len(p8), len(p16)) or (len(p8) == len(p16) and ia["bits"] == 16)
+        assert ia["bits"] == (8 if len(p8) < len(p16) else 16)
+        assert (sp.unpack_ragged(auto, K, N, DELTA, 16, ia["bits"]) == W).all()
+    # the densest of them is the case the detours are for: nearly all gaps fit, a few do not
+    assert ia["bits"] == 8 and auto[:4].tobytes() == b"SPTS" and len(auto) < 0.6 * len(p16)
 
 
 def lds_passes(tasks_bytes, K, N, split, n_task, n_max, shift):

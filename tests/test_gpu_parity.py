@@ -264,9 +264,11 @@ def test_delta_ragged_sparse_and_16bit(K, N, S, splits):
     for split in splits:
         w = sp.Weights.upload_delta(pos, neg, K, split)
         bits = w.info["delta_bits"]
-        assert bits == sp.delta_bits(pos, neg, split)
+        # byte gaps where every gap of the sorted lists fits; else 16-bit gaps, or byte gaps again with the long ones
+        # walked over zero slots of the tile, whichever stream is smaller
+        assert bits == sp.delta_bits(pos, neg, split) or (bits == 8 and w.info["stones"] == 1)
         for M in (1, 4, 5):
-            say("delta", K, N, S, "split", split, "bits", bits, "M", M)
+            say("delta", K, N, S, "split", split, "bits", bits, "stones", w.info["stones"], "M", M)
             X = x_i8(S + M, M, K)
             assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 4)).all(), (split, M)
         Xh = oracle.make_x_normal(split, 2, K, np.float16)
