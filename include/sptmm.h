@@ -131,8 +131,13 @@ int sptmm_pack_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N
  * SPTMM_KIND_U16 (split_k 8..256) or SPTMM_KIND_DELTA (split_k 8..64).  The
  * stream opens with one entry count per wavefront task; a task pads its shorter
  * lists with entries on the zero rows K..K+63 that the activation tile keeps;
- * K + 64 must fit 16 bits.  *bits (gap streams): in 0 = pick 8 when every gap fits a byte,
- * else 16; out the width used.  _bytes returns the stream size (0 on error);
+ * K + 64 must fit 16 bits.  *bits (gap streams): in 0 = pick, 8 or 16 = exactly that; out the
+ * width used.  Byte gaps are signed (+-127 rows).  Where some gap of a lane's run is longer --
+ * the reference's delta layout narrows every gap to u8 unchecked, main.cu:376-394 -- an 8-bit
+ * stream holds positions in a tile that keeps 16 zero slots behind every 112 rows (preamble
+ * magic "SPTS" instead of "SPTR", sptmm_winfo.stones) and walks the gap over zero slots: entries
+ * that add nothing, at most one per 113 positions.  bits = 0 takes that stream when it is
+ * smaller than 16-bit gaps throughout, else 16.  _bytes returns the stream size (0 on error);
  * *read_bytes is what one GEMV reads of it (tasks sit at a fixed stride). */
 size_t sptmm_pack_ragged_bytes(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int *bits, size_t *read_bytes,
                                int *n_min, int *n_max, uint64_t *nnz);
@@ -183,7 +188,10 @@ int sptmm_device_init(int device, sptmm_devinfo *out);
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 /* Gap stream scheduled for calls with `rows` activation rows (sptmm_pack_delta_rows): rows = 1 is
- * the stream for GEMVs (int8, M = 1); 0 = no preference (as sptmm_weights_upload_delta). */
+ * the stream for GEMVs (int8, M = 1); 0 = no preference (as sptmm_weights_upload_delta).
+ * Byte gaps where every gap fits; else the smaller of 16-bit gaps and the 8-bit stream that
+ * walks long gaps over zero slots of the tile (sptmm_pack_ragged; info.ragged and info.stones
+ * are 1 then, info.S stays S). */
 int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int rows, sptmm_weights **out);
 int sptmm_weights_upload_i2s(const int8_t *W_colmajor, int K, int N, sptmm_weights **out);
 /* Any ternary matrix -> device stream of the given kind (ragged u16 lists,
