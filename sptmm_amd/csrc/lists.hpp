@@ -703,10 +703,16 @@ struct ListsBody {
         int n_ahead = p.n_lane;
         if constexpr (VAR) n_ahead = counts[task < p.tasks ? task : 0];
 
-        // 2. ... then the first rounds of the first task's stream ...
+        // 2. ... then the first rounds of the first task's stream (gap streams: and the rows its lanes start from) ...
         Round buf[NB];
+        u32 headp = 0, headq = 0;
         {
-            const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
+            const uint8_t *tb = tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes;
+            const uint4 *wp = reinterpret_cast<const uint4 *>(tb + HDR) + lane;
+            if constexpr (GAPS) {
+                headp = reinterpret_cast<const unsigned short *>(tb)[lane];
+                headq = reinterpret_cast<const unsigned short *>(tb)[64 + lane];
+            }
             if constexpr (RF > 0) {
 #pragma unroll
                 for (int i = 0; i < (RF < EARLY ? RF : EARLY); ++i) buf[i] = load_round(wp, i);
@@ -827,10 +833,21 @@ struct ListsBody {
             const uint4 *wp = reinterpret_cast<const uint4 *>(tb + HDR) + lane;
             u32 runp = 0, runq = 0;
             int n_lane = p.n_lane;
+            // AHEAD: while a task is walked, the next one's first rows and rounds are requested into the registers that
+            // come free, so a wavefront that walks several tasks never waits with nothing in flight.  Four int8 rows
+            // on gap streams only (tasks of one length, straight-line path), where it pays: headline shape, 32 GEMVs per
+            // launch, 10 tasks per wavefront 2.00 -> 1.88 us per GEMV.  Measured and left out: eight int8 rows (2.09 ->
+            // 2.29 us), four fp16 rows (2.18 -> 2.56 us), byte rows (1.70 -> 1.79 us), u16 lists (3.2 -> 13.6 us at M=4).
+            constexpr bool AHEAD = RF != 0 && !VAR && !QUANT && MT == 4 && sizeof(Act) == 1 && MODE != 0;
+            const int task_next = task + task_step;
+            const uint8_t *tb_next = tasks_base + (size_t)(task_next < p.tasks ? task_next : 0) * task_bytes;
             if constexpr (GAPS) {
-                const unsigned short *rs = reinterpret_cast<const unsigned short *>(tb);
-                runp = (u32)rs[lane] << (Fl::GAP8 ? 0 : SH);
-                runq = (u32)rs[64 + lane] << (Fl::GAP8 ? 0 : SH);
+                if ((!AHEAD || (TWIN && plain)) && it > 0) {
+                    headp = reinterpret_cast<const unsigned short *>(tb)[lane];
+                    headq = reinterpret_cast<const unsigned short *>(tb)[64 + lane];
+                }
+                runp = headp << (Fl::GAP8 ? 0 : SH);
+                runq = headq << (Fl::GAP8 ? 0 : SH);
                 if constexpr (is_byte_rows<Act>()) runp += lds_address(smem), runq += lds_address(smem);
             }
             if constexpr (VAR) {
@@ -849,7 +866,7 @@ struct ListsBody {
             acc.init(p.logL);
 
             if constexpr (RF != 0) {
-                if (it > 0) {
+                if (!AHEAD && it > 0) {
 #pragma unroll
                     for (int i = 0; i < NR; ++i) buf[i] = load_round(wp, i);
                 }
@@ -922,8 +939,21 @@ struct ListsBody {
                     if (base + i < R) eat(smem, buf[i], runp, runq, acc);
                 }
             } else {
+                if (AHEAD && it + 1 < p.iters) {
+                    if constexpr (GAPS) {
+                        headp = reinterpret_cast<const unsigned short *>(tb_next)[lane];
+                        headq = reinterpret_cast<const unsigned short *>(tb_next)[64 + lane];
+                    }
+                    const uint4 *wn = reinterpret_cast<const uint4 *>(tb_next + HDR) + lane;
 #pragma unroll
-                for (int i = 0; i < NR; ++i) eat(smem, buf[i], runp, runq, acc);
+                    for (int i = 0; i < NR; ++i) {
+                        eat(smem, buf[i], runp, runq, acc);
+                        buf[i] = load_round(wn, i);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) eat(smem, buf[i], runp, runq, acc);
+                }
                 if constexpr (XMAX > 0) {
 #pragma unroll
                     for (int x = 0; x < XMAX; ++x)

@@ -682,3 +682,45 @@ def test_timing_entry_point_leaves_the_results_of_its_launches(mode, outputs):
         o.free()
     for o in ws:
         o.free()
+
+
+@pytest.mark.parametrize("K,N,S,split,count,M", [
+    (6912, 2560, 4096, 32, 32, 4),    # ten tasks per wavefront: the next task's rounds are requested while one is walked
+    (6912, 2560, 4096, 32, 5, 3),
+    (6912, 2560, 4096, 16, 7, 4),     # eight rounds per task
+    (2560, 6912, 1536, 16, 32, 4),    # three rounds
+    (6912, 2560, 4160, 32, 9, 2),     # four rounds and a one-entry tail
+])
+def test_gap_stream_four_rows_batched_with_many_tasks_per_wavefront(K, N, S, split, count, M):
+    sp.device_init(0)
+    _, pos, neg = matrix(K, N, S)
+    w = sp.Weights.upload_delta(pos, neg, K, split)
+    ws = [w] + [w.clone() for _ in range(min(count, 3) - 1)]
+    ws = [ws[i % len(ws)] for i in range(count)]
+    Xs = [x_i8(300 + i, M, K) for i in range(count)]
+    xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
+    cb = [sp.DeviceBuffer(4 * M * N) for _ in range(count)]
+    for c in cb:
+        c.fill(0xEE)
+    st = sp.Stream()
+    say("gap stream, four rows, batched", K, N, S, split, count, M)
+    sp.gemv_i8_batched(ws, xb, cb, M, st)
+    st.sync()
+    for i in range(count):
+        assert (cb[i].to_numpy(np.int32, (M, N)) == oracle.sptmm_i8_mt(Xs[i], pos, neg, 8)).all(), i
+    for o in xb + cb:
+        o.free()
+
+
+def test_gap_stream_four_rows_single_launch_with_several_tasks_per_wavefront():
+    """A lone launch walks more than one task per wavefront when the tasks outnumber the wavefronts the chip holds."""
+    sp.device_init(0)
+    K, N, S = 2560, 13824, 1536
+    _, pos, neg = matrix(K, N, S)
+    for split in (16, 32, 64):
+        w = sp.Weights.upload_delta(pos, neg, K, split)
+        for M in (4, 2):
+            say("gap stream, four rows, many tasks", split, M)
+            X = x_i8(77 + M, M, K)
+            assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), (split, M)
+        w.free()
