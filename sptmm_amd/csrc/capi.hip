@@ -231,7 +231,7 @@ int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, in
         if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
         int bits = sptmm_delta_bits(pos, neg, N, S, split_k);
         if (bits < 0) return bits;
-        if (bits == 16 && K + 64 <= 65535) {
+        if (bits == 16 && K + 64 <= 65535 && (size_t)K * N <= ((size_t)1 << 30)) {  // (the detour builder wants the dense matrix: 1 GiB at most)
             // Some gap is too long for a byte (the reference narrows every gap to u8 unchecked, main.cu:376-394).  The
             // builder for arbitrary matrices can walk long gaps over zero slots of the tile; take its stream where
             // that is smaller than 16-bit gaps throughout.

@@ -34,6 +34,7 @@ def cases(seed, count):
 
 @pytest.mark.parametrize("kind,splits", [(sp.KIND_U16, (8, 16, 32, 64, 128, 256)), (sp.KIND_DELTA, (8, 16, 32, 64))])
 def test_ragged_random_shapes(kind, splits):
+    detours = 0  # gap streams that walk long gaps over zero slots of the tile
     for i, (K, N, pp, pn, M, seed) in enumerate(cases(20240 + kind, 40)):
         W = sp.generate_ternary_iid(K, N, seed, pp, pn)
         X = oracle.make_x_i8(seed ^ 0x55, M, K)
@@ -41,10 +42,12 @@ def test_ragged_random_shapes(kind, splits):
         split = splits[i % len(splits)]
         print("random ragged", kind, "K", K, "N", N, "p", round(pp, 3), round(pn, 3), "M", M, "split", split, flush=True)
         sys.stdout.flush()
-        w = sp.Weights.upload_dense(W, kind, split)
+        w = sp.Weights.upload_dense(W, kind, split, rows=1 if kind == sp.KIND_DELTA and i % 3 == 0 else 0)
+        detours += w.info["stones"]
         got = w.matmul(X)
         w.free()
         assert (got == want).all(), (K, N, pp, pn, M, split)
+    assert kind == sp.KIND_U16 or detours >= 3, detours
 
 
 def test_balanced_random_shapes():
