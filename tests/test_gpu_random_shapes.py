@@ -73,3 +73,51 @@ def test_balanced_random_shapes():
             w = sp.Weights.upload_delta(pos, neg, K, split)
             assert (w.matmul(X) == want).all(), ("delta", K, N, half, split, M, w.info["delta_bits"])
             w.free()
+
+
+def test_batched_random_shapes():
+    """One launch of 1-40 GEMVs of one random shape, every stream kind and row count: each output equals the oracle's.
+    Batched launches regroup their tasks (up to 16 per wavefront, workgroups of up to 16 wavefronts); the shapes here
+    make task counts that do not divide evenly."""
+    rng = np.random.default_rng(99)
+    kinds = ("u16", "gap", "gap1", "dense gap", "dense gap1", "wide u16", "wide gap", "i2s")
+    for i in range(48):
+        kind = kinds[i % len(kinds)]
+        K = 16 * int(rng.integers(4, 500))
+        N = 16 * int(rng.integers(1, 60))
+        split = int(rng.choice([8, 16, 32, 64]))
+        M = int(rng.choice([1, 1, 2, 4, 5, 8, 9, 16]))
+        count = int(rng.choice([1, 2, 4, 5, 7, 8, 13, 32, 33, 40]))
+        dens = float(rng.choice([0.03, 0.1, 0.3, 0.6]))
+        if kind in ("u16", "gap", "gap1"):
+            n_lane = max(1, int(dens * K / 2 / split))
+            S = 2 * split * n_lane
+            if S >= K:
+                S = 2 * split * max(1, (K - 16) // (2 * split))
+            W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+            w = (sp.Weights.upload_u16(pos, neg, K, split) if kind == "u16" else
+                 sp.Weights.upload_delta(pos, neg, K, split, rows=1 if kind == "gap1" else 0))
+        else:
+            W = sp.generate_ternary_iid(K, N, int(rng.integers(0, 2**31)), dens * 0.6, dens * 0.4)
+            w = (sp.Weights.upload_dense(W, sp.KIND_DELTA, split, rows=1 if kind == "dense gap1" else 0) if kind.startswith("dense") else
+                 sp.Weights.upload_wide(W, sp.KIND_U16 if kind == "wide u16" else sp.KIND_DELTA, split) if kind.startswith("wide") else
+                 sp.Weights.upload_i2s(W))
+        print("random batched", kind, "K", K, "N", N, "split", split, "M", M, "count", count, "dens", dens, flush=True)
+        sys.stdout.flush()
+        ws = [w] + [w.clone() for _ in range(min(count, 3) - 1)]
+        ws = [ws[j % len(ws)] for j in range(count)]
+        Xs = [oracle.make_x_i8(1000 * i + j, M, K) for j in range(min(count, 4))]
+        xb = [sp.DeviceBuffer.from_numpy(x) for x in Xs]
+        cb = [sp.DeviceBuffer(4 * M * N) for _ in range(count)]
+        for c in cb:
+            c.fill(0xEE)
+        st = sp.Stream()
+        sp.gemv_i8_batched(ws, [xb[j % len(xb)] for j in range(count)], cb, M, st)
+        st.sync()
+        want = [oracle.dense_i8(x, W) for x in Xs]
+        for j in range(count):
+            assert (cb[j].to_numpy(np.int32, (M, N)) == want[j % len(want)]).all(), (kind, K, N, split, M, count, j)
+        for o in xb + cb:
+            o.free()
+        for o in set(ws):
+            o.free()
