@@ -1190,14 +1190,17 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // (K=13824 N=5120, M=8, 10 -> 12 wavefronts: gap stream 48 -> 55 % of HBM peak, u16 lists level)
     // -- and the largest workgroup does best: four wavefronts per SIMD, fewer workgroups staging (same shape, 12 -> 16
     // wavefronts: gap stream 9.95 -> 9.46 us per GEMV, u16 lists 14.0 -> 13.8 us)
-    if (MT == 8 && a.batch >= 4 && a.W == 1 && max_waves >= 4) wpb = max_waves / 4 * 4;
+    // (also where two tiles would fit a compute unit: the registers of an eight-row kernel allow 16 wavefronts per CU either
+    // way, and one workgroup of 16 stages the tile once -- K=6912 N=2560, M=8, 8 -> 16 wavefronts: u16 3.65 -> 3.40 us, gap
+    // stream level at 2.14-2.40 us from box to box)
+    if (MT == 8 && a.batch >= 4 && a.W == 1 && !a.quant) wpb = lists_max_waves<Act, MT, false>() / 4 * 4;
     // four-row tiles on gap streams, batched, tile small enough for several workgroups per CU: eight wavefronts
     // (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824 five do better)
     if (MT == 4 && MODE != 0 && a.batch >= 4 && a.W == 1 && tile <= 40 * 1024 && max_waves >= 8) wpb = 8;
     // four fp16 rows (sums on the matrix unit, 56 KB tile at K=6912), batched: eight wavefronts as well
     // (headline shape, 5 -> 8: u16 lists 69 -> 81 % of HBM peak, gap stream 39 -> 53 %)
     if (MT == 4 && sizeof(Act) == 2 && a.batch >= 4 && a.W == 1 && max_waves >= 8) wpb = 8;
-    if (tune_wpb > 0 && tune_wpb <= max_waves && tune_wpb % a.W == 0) wpb = tune_wpb;
+    if (tune_wpb > 0 && tune_wpb <= (a.quant ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>()) && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
     int grid_x = blocks < slots ? blocks : slots;
