@@ -411,6 +411,11 @@ static int launch_i2s_mfma(const GemvArgs &a, hipStream_t st)
     if (a.batch >= 4) {
         ct = xj >= 3 ? 8 : 4;
         waves = 4;
+        // ... as long as the launch still has workgroups enough: four per compute unit, eight where a workgroup's share
+        // of K is short (K=2560, 32 GEMVs per launch: N=640 4 -> 1 tiles 0.200 -> 0.154 us per GEMV, N=2560 4 -> 2 tiles
+        // 0.379 -> 0.355 us; N=6912 stays at 4: 0.82 against 0.89 / 1.05 us)
+        const long need = (long)(a.compute_units > 0 ? a.compute_units : 256) * (rounds >= 16 ? 4 : 8);
+        while (ct > 1 && (long)a.batch * (groups / ct) < need) ct /= 2;
     } else {
         while (ct < 4 && groups / (2 * ct) >= 160) ct *= 2;
     }
