@@ -414,7 +414,10 @@ int sptmm_choose_split_k(int kind, int N, int S, int compute_units)
 {
     // Measured on MI355X over the decoder-layer shapes, K = 2560 ... 13824, N = 128 ... 13824: a lane does best with
     // some 30 to 70 entries per sign (fewer and the per-task overhead shows, more and too few tasks are in flight),
-    // and a launch wants at least two tasks per compute unit -- small N pays for that with shorter lanes, down to 8.
+    // and a launch wants at least two tasks per compute unit -- small N pays for that with shorter lanes, down to 24
+    // entries: below that a lone launch gains nothing any more and a batched one, which fills the chip with other
+    // GEMVs, loses (K=2560 N=640 S=1536, split 32 / 64: alone 3.52 / 3.77 us HBM-cold, 32 per launch 0.33 / 0.41 us
+    // per GEMV; K=3072 N=768 S=256, split 8 / 16: 3.64 / 3.69 and 0.19 / 0.26 us).
     const int max_split = kind == SPTMM_KIND_U16 ? 256 : 64;
     if ((kind != SPTMM_KIND_U16 && kind != SPTMM_KIND_DELTA) || N <= 0 || S <= 0 || S % 2) return fail(SPTMM_ERR_INVALID, "no split for this kind or shape");
     const int half = S / 2, cus = compute_units > 0 ? compute_units : 256;
@@ -427,7 +430,7 @@ int sptmm_choose_split_k(int kind, int N, int S, int compute_units)
             if (half / s <= 72) break;
         }
     if (!pick) return fail(SPTMM_ERR_INVALID, "Wrong SPLIT Size: no split_k in 8..%d divides S/2 = %d with N = %d", max_split, half, N);
-    while (tasks(pick) < 2L * cus && valid(2 * pick) && half / (2 * pick) >= 8) pick *= 2;
+    while (tasks(pick) < 2L * cus && valid(2 * pick) && half / (2 * pick) >= 24) pick *= 2;
     return pick;
 }
 

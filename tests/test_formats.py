@@ -363,10 +363,11 @@ def test_non_positive_shapes_are_refused_before_anything_is_read():
 
 def test_automatic_split_k_is_valid_and_follows_the_measured_rule():
     """split_k = 0 in the upload calls: 30-70 entries per lane where the matrix is wide enough for two tasks per
-    compute unit, shorter lanes (down to 8 entries) where it is not; always a split the packers accept."""
-    want = {(sp.KIND_U16, 2560, 4096): 32, (sp.KIND_DELTA, 2560, 4096): 32, (sp.KIND_U16, 640, 1536): 64, (sp.KIND_U16, 2560, 1536): 16,
-            (sp.KIND_U16, 6912, 1536): 16, (sp.KIND_U16, 5120, 8320): 64, (sp.KIND_DELTA, 5120, 8320): 64, (sp.KIND_U16, 128, 4096): 256,
-            (sp.KIND_DELTA, 128, 4096): 64, (sp.KIND_U16, 2560, 4160): 32}
+    compute unit, shorter lanes (down to 24 entries) where it is not; always a split the packers accept."""
+    want = {(sp.KIND_U16, 2560, 4096): 32, (sp.KIND_DELTA, 2560, 4096): 32, (sp.KIND_U16, 640, 1536): 32, (sp.KIND_U16, 2560, 1536): 16,
+            (sp.KIND_U16, 6912, 1536): 16, (sp.KIND_U16, 5120, 8320): 64, (sp.KIND_DELTA, 5120, 8320): 64, (sp.KIND_U16, 128, 4096): 64,
+            (sp.KIND_DELTA, 128, 4096): 64, (sp.KIND_U16, 2560, 4160): 32, (sp.KIND_U16, 640, 4096): 64, (sp.KIND_U16, 768, 256): 8,
+            (sp.KIND_DELTA, 768, 512): 8}
     for (kind, N, S), split in want.items():
         assert sp.choose_split_k(kind, N, S, 256) == split, (kind, N, S)
     rng = np.random.default_rng(3)
