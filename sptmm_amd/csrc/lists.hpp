@@ -660,8 +660,9 @@ struct ListsBody {
         constexpr int NR = RF > 0 ? RF : 0;               // full rounds of the straight-line body (RF == -1: none, tails only)
         constexpr int NB = RF > 0 ? RF : RF == 0 ? RING : 1;
         // stepping-stone streams: item i (16 rows) goes to item i + i/7 of the tile, every eighth item stays zero
-        const int tile_rows = p.stones ? STONE_BLOCK * ((p.K + STONE_ROWS - 1) / STONE_ROWS) : p.K;
-        auto place = [&](int item) { return p.stones ? item + item / (STONE_ROWS / 16) : item; };
+        const bool stones = Fl::GAP8 && VAR && p.stones;  // (only ragged 8-bit gap streams come with zero slots: nothing of this in the other kernels)
+        const int tile_rows = stones ? STONE_BLOCK * ((p.K + STONE_ROWS - 1) / STONE_ROWS) : p.K;
+        auto place = [&](int item) { return stones ? item + item / (STONE_ROWS / 16) : item; };
         A *part = reinterpret_cast<A *>(smem + (size_t)(tile_rows + ZROWS) * SLOT);
         const int tid = threadIdx.x, nt = blockDim.x;
         const int lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
@@ -800,7 +801,7 @@ struct ListsBody {
         // rows K.. read as zero
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
             reinterpret_cast<u32 *>(smem + (size_t)tile_rows * SLOT)[i] = 0u;
-        if (p.stones) {
+        if (stones) {
             // the zero slots inside the tile: every eighth item, and what the last block holds beyond row K-1
             constexpr int DW = 4 * SLOT;  // dwords per item
             for (int i = tid; i < tile_rows / 16 * DW; i += nt) {
