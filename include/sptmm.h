@@ -213,7 +213,9 @@ void sptmm_weights_free(sptmm_weights *w);
  * main.cu:242-509, repeated by every run of the reference) happens once: a
  * fixed header (shape, encoding, checksum) followed by the device stream as it
  * is.  load checks the header against the stream size, the checksum and, for
- * ragged streams, the count table, before anything reaches the device. */
+ * ragged and wide streams, the count tables (wide: every K-tile's offset, stride
+ * and counts, and that its K-tile fits this device's LDS: SPTMM_ERR_UNSUPPORTED
+ * otherwise), before anything reaches the device. */
 int sptmm_weights_save(const sptmm_weights *w, const char *path);
 int sptmm_weights_load(const char *path, sptmm_weights **out);
 int sptmm_weights_info(const sptmm_weights *w, sptmm_winfo *out);

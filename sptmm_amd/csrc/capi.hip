@@ -427,7 +427,6 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
 {
     return guarded([&]() -> int {
         if (!w || !path) return fail(SPTMM_ERR_INVALID, "null pointer");
-        if (w->wide) return fail(SPTMM_ERR_UNSUPPORTED, "wide streams are tied to the LDS size of the device they were packed for and are not saved");
         std::vector<uint8_t> host(w->bytes);
         HIP_TRY(hipMemcpy(host.data(), w->dev, w->bytes, hipMemcpyDeviceToHost));
         FileHeader h{};
@@ -436,7 +435,8 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
         h.version = 2;
         const sptmm_winfo &i = w->info;
         const Geometry &g = w->geo;
-        h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = i.ragged;
+        // ragged: 0 balanced, 1 ragged, 2 wide (K-tiled; the stream's own 512-byte header holds the tiles' offsets and counts)
+        h.kind = i.kind, h.K = i.K, h.N = i.N, h.S = i.S, h.split_k = i.split_k, h.delta_bits = i.delta_bits, h.ragged = w->wide ? 2 : i.ragged;
         h.half = g.half, h.L = g.L, h.G = g.G, h.W = g.W, h.n_lane = g.n_lane, h.tasks = g.tasks;
         h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max;
         h.index_shift = i.kind == SPTMM_KIND_DELTA ? (w->byte_rows ? 2 : 0) : w->index_shift;
@@ -472,6 +472,13 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
                 const bool gaps = h.kind == SPTMM_KIND_DELTA;
                 if (gaps ? (h.delta_bits != 8 && h.delta_bits != 16) : h.delta_bits != 0) {
                     rc = fail(SPTMM_ERR_INVALID, "%s: bad gap width", path);
+                } else if (h.ragged == 2) {
+                    // wide stream: shape and geometry here, the K-tiles' tables once the stream is in memory
+                    if (h.K <= 0 || h.N <= 0 || h.K % 16 || h.N % 16 || h.K >= 65536 || h.split_k > 64 || make_ragged_geometry(h.N, h.split_k, 64, &g) ||
+                        h.index_shift != 0 || h.task_stride != 0 || h.counts_bytes != 0 || h.stream_bytes < 1024 || h.stream_bytes > 0xffffffffull)
+                        rc = fail(SPTMM_ERR_INVALID, "%s: inconsistent wide stream header", path);
+                    else
+                        want = (size_t)h.stream_bytes;
                 } else if (h.ragged) {
                     const int esz = gaps ? h.delta_bits / 8 : 2;
                     if (h.K <= 0 || h.N <= 0 || h.K % 16 || h.N % 16 || h.K + 64 > 65535 || make_ragged_geometry(h.N, h.split_k, max_split, &g) ||
@@ -513,7 +520,30 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
                     for (int q = 0; q < 4; ++q) memcpy(host.data() + t + (size_t)(16 * q + c) * 16, tile.data() + (size_t)(4 * c + q) * 16, 16);
             }
         }
-        if (h.ragged && (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA)) {
+        WideHeader wh;
+        if (h.ragged == 2) {
+            // every offset, stride and count the kernel follows is checked against the stream and the device's LDS
+            DevCaps caps;
+            if (int crc = device_caps(&caps)) return crc;
+            const int esz = h.kind == SPTMM_KIND_U16 ? 2 : h.delta_bits / 8, hdr = h.kind == SPTMM_KIND_DELTA ? 256 : 0;
+            if (wide_parse_header(host.data(), &wh)) return fail(SPTMM_ERR_INVALID, "%s: not a wide stream", path);
+            bool ok = wh.K == h.K && wh.N == h.N && wh.kind == h.kind && wh.bits == h.delta_bits && wh.split_k == h.split_k && wh.k_tile > 0 &&
+                      wh.k_tile % 16 == 0 && wh.k_tile + 64 <= 16383 && wh.phases == (h.K + wh.k_tile - 1) / wh.k_tile;
+            if (ok && (size_t)(wh.k_tile + 64) * 16 + 64 > (size_t)caps.lds)
+                return fail(SPTMM_ERR_UNSUPPORTED, "%s: K-tiles of %d rows were packed for a larger LDS than this device's %d bytes", path, wh.k_tile, caps.lds);
+            const size_t table = ragged_counts_bytes(h.tasks);
+            for (int p = 0; ok && p < wh.phases; ++p) {
+                const size_t off = wh.offset[p], stride = wh.stride[p];
+                ok = off >= 512 && off % 256 == 0 && wh.n_min[p] >= 1 && wh.n_max[p] >= wh.n_min[p] && wh.n_max[p] <= 65535 &&
+                     stride == hdr + (size_t)128 * esz * wh.n_max[p] && off + table + stride * h.tasks <= host.size();
+                if (!ok) break;
+                const uint32_t *pre = (const uint32_t *)(host.data() + off);
+                const uint16_t *counts = (const uint16_t *)(host.data() + off + 16);
+                ok = pre[0] == RAGGED_MAGIC && pre[1] == (uint32_t)h.tasks && pre[2] == (uint32_t)wh.n_max[p] && pre[3] == (uint32_t)wh.n_min[p];
+                for (int t = 0; ok && t < h.tasks; ++t) ok = counts[t] >= wh.n_min[p] && counts[t] <= wh.n_max[p];
+            }
+            if (!ok) return fail(SPTMM_ERR_INVALID, "%s: corrupt wide stream tables", path);
+        } else if (h.ragged && (h.kind == SPTMM_KIND_U16 || h.kind == SPTMM_KIND_DELTA)) {
             // the per-task counts are what the kernel trusts most: keep them inside [n_min, n_max]
             const uint32_t *pre = (const uint32_t *)host.data();
             const uint16_t *counts = (const uint16_t *)(host.data() + 16);
@@ -524,8 +554,14 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         }
         sptmm_weights *w = new (std::nothrow) sptmm_weights();
         if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
-        w->info = sptmm_winfo{h.kind, h.K, h.N, h.S, h.split_k, h.delta_bits, h.read_bytes, h.ragged, h.nnz};
+        w->info = sptmm_winfo{h.kind, h.K, h.N, h.S, h.split_k, h.delta_bits, h.read_bytes, h.ragged ? 1 : 0, h.nnz};
         w->geo = Geometry{h.N, h.half, h.split_k, h.L, h.G, h.W, h.n_lane, h.tasks};
+        if (h.ragged == 2) {
+            w->wide = true;
+            w->wh = wh;
+            w->info.k_tile = wh.k_tile;
+            return finish_upload(w, host, out);
+        }
         w->task_stride = h.task_stride;
         w->counts_bytes = h.counts_bytes;
         w->n_min = h.n_min;

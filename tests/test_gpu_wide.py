@@ -147,9 +147,6 @@ def test_refusals():
     with pytest.raises(sp.SptmmError) as e:
         w.gemv_q8(xb, 1, 1, 1.0, cb)
     assert e.value.code == -2
-    with pytest.raises(sp.SptmmError) as e:
-        w.save("/tmp/never_written.sptmm")
-    assert e.value.code == -2
     with pytest.raises(sp.SptmmError):
         sp.Weights.upload_wide(W, sp.KIND_I2S, 32)
     for o in (w, xb, cb):

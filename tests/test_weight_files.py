@@ -33,6 +33,7 @@ def test_save_load_round_trip_every_encoding(tmp_path):
     K, N, S = 2560, 640, 1536
     W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
     Wi = sp.generate_ternary_iid(K, N, 3, 0.3, 0.3)
+    Ws = sp.generate_ternary_iid(K, N, 4, 0.03, 0.03)
     X = oracle.make_x_i8(7, 4, K)
     makers = {
         "u16": lambda: sp.Weights.upload_u16(pos, neg, K, 32),
@@ -41,6 +42,9 @@ def test_save_load_round_trip_every_encoding(tmp_path):
         "i2s": lambda: sp.Weights.upload_i2s(W),
         "ragged_u16": lambda: sp.Weights.upload_dense(Wi, sp.KIND_U16, 32),
         "ragged_delta": lambda: sp.Weights.upload_dense(Wi, sp.KIND_DELTA, 16),
+        "ragged_sparse_delta": lambda: sp.Weights.upload_dense(Ws, sp.KIND_DELTA, 16, rows=1),   # 8-bit gaps over zero slots
+        "ragged_wide_u16": lambda: sp.Weights.upload_wide(Wi, sp.KIND_U16, 32),
+        "ragged_wide_delta": lambda: sp.Weights.upload_wide(Wi, sp.KIND_DELTA, 16),
     }
     for name, mk in makers.items():
         print("weight file", name, flush=True)
@@ -53,7 +57,7 @@ def test_save_load_round_trip_every_encoding(tmp_path):
         v = sp.Weights.load(path)
         assert v.info == w.info and v.nbytes == w.nbytes
         assert (v.matmul(X) == want).all()
-        assert (want == oracle.dense_i8(X, Wi if name.startswith("ragged") else W)).all()
+        assert (want == oracle.dense_i8(X, Ws if "sparse" in name else Wi if name.startswith("ragged") else W)).all()
         w.free()
         v.free()
         # one flipped stream byte, a truncated file and trailing bytes are all refused
@@ -111,3 +115,39 @@ def test_version_1_i2s_file_is_retiled_on_load(tmp_path):
     v = sp.Weights.load(p1)
     assert (v.matmul(X) == oracle.dense_i8(X, W)).all()
     v.free()
+
+
+@pytest.mark.gpu
+def test_wide_file_with_a_bad_table_is_refused_although_its_checksum_holds(tmp_path):
+    """The K-tiles' offsets, strides and per-task counts are what the kernel follows: a file whose checksum was
+    recomputed over a damaged table must still not load."""
+    sp.device_init(0)
+    K, N = 2560, 64
+    W = sp.generate_ternary_iid(K, N, 5, 0.3, 0.3)
+    w = sp.Weights.upload_wide(W, sp.KIND_DELTA, 32)
+    path = str(tmp_path / "wide.sptmm")
+    w.save(path)
+    X = oracle.make_x_i8(3, 16, K)
+    v = sp.Weights.load(path)
+    assert v.info == w.info and v.info["k_tile"] > 0 and (v.matmul(X) == oracle.dense_i8(X, W)).all()
+    v.free()
+    w.free()
+    raw = bytearray(open(path, "rb").read())
+    hdr = np.frombuffer(bytes(raw[120:120 + 512]), np.uint32)
+    off = int(hdr[8])
+    damages = {
+        "count above n_max": (120 + off + 16, (65535).to_bytes(2, "little")),
+        "offset past the stream": (120 + 4 * 8, (len(raw)).to_bytes(4, "little")),
+        "stride": (120 + 4 * 9, (int(hdr[9]) + 128).to_bytes(4, "little")),
+        "k_tile": (120 + 4 * 2, (16320).to_bytes(4, "little")),
+        "phases": (120 + 4 * 1, (3).to_bytes(4, "little")),
+    }
+    for what, (at, val) in damages.items():
+        bad = bytearray(raw)
+        bad[at:at + len(val)] = val
+        bad[112:120] = bytes(8)                      # the checksum covers the header with this field zero, then the stream
+        bad[112:120] = _fnv1a(bytes(bad)).to_bytes(8, "little")
+        open(path, "wb").write(bytes(bad))
+        with pytest.raises(sp.SptmmError) as e:
+            sp.Weights.load(path)
+        assert "checksum" not in str(e.value), (what, str(e.value))
