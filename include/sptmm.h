@@ -63,7 +63,7 @@ typedef struct sptmm_winfo {
     int row_bytes;   /* 8-bit gap streams: bytes per row of the activation tile the visiting order was scheduled for,
                       * 1 (sptmm_*_rows with rows = 1) or 4; 0 for every other stream */
     int stones;      /* 1: 8-bit gap stream of a matrix too sparse for byte gaps throughout -- the activation tile keeps 16 zero
-                      * slots behind every 112 rows, the stream holds tile positions, and a gap of more than 127 positions
+                      * slots behind every 96 rows, the stream holds tile positions, and a gap of more than 127 positions
                       * is walked over zero slots (entries that add nothing); 0 for every other stream */
 } sptmm_winfo;
 
@@ -134,9 +134,9 @@ int sptmm_pack_delta_rows(const uint16_t *pos, const uint16_t *neg, int K, int N
  * K + 64 must fit 16 bits.  *bits (gap streams): in 0 = pick, 8 or 16 = exactly that; out the
  * width used.  Byte gaps are signed (+-127 rows).  Where some gap of a lane's run is longer --
  * the reference's delta layout narrows every gap to u8 unchecked, main.cu:376-394 -- an 8-bit
- * stream holds positions in a tile that keeps 16 zero slots behind every 112 rows (preamble
+ * stream holds positions in a tile that keeps 16 zero slots behind every 96 rows (preamble
  * magic "SPTS" instead of "SPTR", sptmm_winfo.stones) and walks the gap over zero slots: entries
- * that add nothing, at most one per 113 positions.  bits = 0 takes that stream when it is
+ * that add nothing, at most one per 97 positions.  bits = 0 takes that stream when it is
  * smaller than 16-bit gaps throughout, else 16.  _bytes returns the stream size (0 on error);
  * *read_bytes is what one GEMV reads of it (tasks sit at a fixed stride). */
 size_t sptmm_pack_ragged_bytes(const int8_t *W_colmajor, int K, int N, int kind, int split_k, int *bits, size_t *read_bytes,

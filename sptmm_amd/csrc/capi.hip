@@ -24,7 +24,7 @@ struct sptmm_weights {
     int n_min = 0, n_max = 0;
     int index_shift = 0;  // u16 streams: fields are row << index_shift
     bool byte_rows = false;  // 8-bit gap stream scheduled for a tile of one byte per row
-    bool stones = false;     // 8-bit gap stream of tile positions (zero slots behind every 112 rows of the tile)
+    bool stones = false;     // 8-bit gap stream of tile positions (zero slots behind every 96 rows of the tile)
     bool wide = false;    // wide stream (K-tiled, 16-byte slots): `wh` describes it
     WideHeader wh;
 };

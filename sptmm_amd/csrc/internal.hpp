@@ -123,11 +123,13 @@ int ragged_index_shift(int K);
 // ragged streams open with a 16-byte preamble {u32 magic, tasks, n_max, n_min} and one u16 entry
 // count per task; the tasks follow at the next multiple of 256 bytes
 constexpr uint32_t RAGGED_MAGIC = 0x52545053u;  // "SPTR"
-// 8-bit gap streams of sparse matrices ("stepping stones"): the activation tile keeps 16 zero slots behind every 112
+// 8-bit gap streams of sparse matrices ("stepping stones"): the activation tile keeps 16 zero slots behind every 96
 // rows, the stream holds tile positions instead of rows, and a gap of more than 127 positions is walked over zero
-// slots, each an entry that adds nothing.  Any 127 consecutive positions hold a zero slot.
+// slots, each an entry that adds nothing.  Any 127 consecutive positions hold a zero slot.  The period of 112 slots
+// moves the zero slots of successive blocks to other LDS banks (a period of 128 would keep them all on the same ones,
+// and lanes that wait on zero slots for the rest of their task would queue there).
 constexpr uint32_t RAGGED_MAGIC_STONES = 0x53545053u;  // "SPTS"
-constexpr int STONE_ROWS = 112, STONE_BLOCK = 128;
+constexpr int STONE_ROWS = 96, STONE_BLOCK = 112;
 inline int stone_blocks(int K) { return (K + STONE_ROWS - 1) / STONE_ROWS; }
 inline int stone_tile_rows(int K) { return STONE_BLOCK * stone_blocks(K); }                 // positions of the tile (zero slots included)
 inline int stone_pos(int row) { return row + (STONE_BLOCK - STONE_ROWS) * (row / STONE_ROWS); }
@@ -164,7 +166,7 @@ struct GemvArgs {
     int compute_units;
     int lds_limit;
     int byte_rows = 0;    // 8-bit gap stream scheduled for a tile of one byte per row (int8, one activation row)
-    int stones = 0;       // 8-bit gap stream of tile positions with zero slots behind every 112 rows (RAGGED_MAGIC_STONES)
+    int stones = 0;       // 8-bit gap stream of tile positions with zero slots behind every 96 rows (RAGGED_MAGIC_STONES)
     int quant = 0;        // 1 / 2: X holds fp16 / bf16 rows, quantised to int8 in the kernel; C receives floats
     float w_scale = 1.f;  // quantising launches: factor applied to every output
     // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each

@@ -475,7 +475,7 @@ struct ListParams {
     int iters;  // tasks each wavefront walks: ceil(tasks / (gridDim.x * waves))
     int quant;      // quantising kernels: X holds 1 = fp16, 2 = bf16 values
     float w_scale;  // quantising kernels: factor applied to every output
-    int stones;     // 8-bit gap streams of tile positions: the tile keeps 16 zero slots behind every 112 rows
+    int stones;     // 8-bit gap streams of tile positions: the tile keeps 16 zero slots behind every 96 rows
 };
 
 // rows of the activation tile in front of its 64 trailing zero rows
@@ -659,7 +659,7 @@ struct ListsBody {
     {
         constexpr int NR = RF > 0 ? RF : 0;               // full rounds of the straight-line body (RF == -1: none, tails only)
         constexpr int NB = RF > 0 ? RF : RF == 0 ? RING : 1;
-        // stepping-stone streams: item i (16 rows) goes to item i + i/7 of the tile, every eighth item stays zero
+        // stepping-stone streams: item i (16 rows) goes to item i + i/6 of the tile, every seventh item stays zero
         const bool stones = Fl::GAP8 && VAR && p.stones;  // (only ragged 8-bit gap streams come with zero slots: nothing of this in the other kernels)
         const int tile_rows = stones ? STONE_BLOCK * ((p.K + STONE_ROWS - 1) / STONE_ROWS) : p.K;
         auto place = [&](int item) { return stones ? item + item / (STONE_ROWS / 16) : item; };
@@ -802,12 +802,14 @@ struct ListsBody {
         for (int i = tid; i < ZROWS * SLOT / 4; i += nt)
             reinterpret_cast<u32 *>(smem + (size_t)tile_rows * SLOT)[i] = 0u;
         if (stones) {
-            // the zero slots inside the tile: every eighth item, and what the last block holds beyond row K-1
-            constexpr int DW = 4 * SLOT;  // dwords per item
-            for (int i = tid; i < tile_rows / 16 * DW; i += nt) {
-                const int j = i / DW;
-                if (j % 8 == 7 || j - j / 8 >= items) reinterpret_cast<u32 *>(smem)[i] = 0u;
-            }
+            // the zero slots inside the tile: the last item of every block, and what the last block holds beyond row K-1
+            constexpr int DW = 4 * SLOT;                // dwords per item
+            constexpr int BI = STONE_BLOCK / 16;        // items per block
+            const int blocks = tile_rows / STONE_BLOCK;
+            u32 *t32 = reinterpret_cast<u32 *>(smem);
+            for (int i = tid; i < blocks * DW; i += nt) t32[((i / DW + 1) * BI - 1) * DW + i % DW] = 0u;
+            const int first_free = place(items - 1) + 1, past = blocks * BI - 1;  // items of the last block without rows
+            for (int i = tid; i < (past - first_free) * DW; i += nt) t32[first_free * DW + i] = 0u;
         }
         // TWIN: one flag per wavefront behind the per-wavefront sums, folded by every thread after the barrier
         u32 *nf_flags = reinterpret_cast<u32 *>(part + waves * MT);

@@ -267,7 +267,8 @@ void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
                 stone_runs(pl, task, sign, n0, rows[sign]);
                 for (int lane = 0; lane < 64; ++lane) {
                     std::vector<uint16_t> &r = rows[sign][lane];
-                    const int rest = r.empty() ? STONE_ROWS : STONE_BLOCK * (r.back() / STONE_BLOCK) + STONE_ROWS;
+                    // (one of the block's 16 zero slots per lane: they lie on different banks)
+                    const int rest = (r.empty() ? STONE_ROWS : STONE_BLOCK * (r.back() / STONE_BLOCK) + STONE_ROWS) + (lane & 15);
                     r.resize(n, (uint16_t)rest);
                 }
             }

@@ -184,8 +184,8 @@ def test_gap_stream_for_single_rows_holds_the_same_matrix_on_other_banks(split):
 
 
 def stone_pos(r):
-    """Position of row r in a tile that keeps 16 zero slots behind every 112 rows."""
-    return r + 16 * (r // 112)
+    """Position of row r in a tile that keeps 16 zero slots behind every 96 rows."""
+    return r + 16 * (r // 96)
 
 
 def walks_of(packed, n_max, table, task, sign):
@@ -204,7 +204,7 @@ def walks_of(packed, n_max, table, task, sign):
 
 @pytest.mark.parametrize("K,N,split,p", [(6912, 32, 32, 0.01), (6912, 32, 16, 0.04), (2560, 64, 8, 0.02), (3072, 48, 16, 0.04), (2560, 16, 64, 0.02)])
 def test_sparse_matrix_walks_long_gaps_over_zero_slots(K, N, split, p):
-    """Gaps of more than 127 rows: an 8-bit stream of tile positions (16 zero slots behind every 112 rows) whose lanes
+    """Gaps of more than 127 rows: an 8-bit stream of tile positions (16 zero slots behind every 96 rows) whose lanes
     step over zero slots.  Every lane visits exactly the positions of its share of the sorted list, plus zero slots
     only; every step fits a signed byte; what unpacks is the matrix."""
     W = sp.generate_ternary_iid(K, N, 5, p, p)
@@ -217,7 +217,7 @@ def test_sparse_matrix_walks_long_gaps_over_zero_slots(K, N, split, p):
     G, L = 64 // split, split
     tasks = N // G
     table = -(-(16 + 2 * tasks) // 256) * 256
-    tile = 128 * -(-K // 112)
+    tile = 112 * -(-K // 96)
     grew = 0
     for task in range(tasks):
         n0 = max(1, max(-(-int((W[task * G + c] == v).sum()) // L) for c in range(G) for v in (1, -1)))
@@ -230,7 +230,7 @@ def test_sparse_matrix_walks_long_gaps_over_zero_slots(K, N, split, p):
                 rows = np.flatnonzero(W[task * G + lane // L] == val)
                 mine = [stone_pos(int(r)) for r in rows[(lane % L) * n0:(lane % L + 1) * n0]]
                 seen = walks[lane]
-                real = sorted(int(x) for x in seen if x % 128 < 112)
+                real = sorted(int(x) for x in seen if x % 112 < 96)
                 assert real == mine, (task, sign, lane)   # every other visit is a zero slot
     assert grew > 0  # some task did need a detour
     # the same stream for tiles of one byte per row: same size, same matrix
