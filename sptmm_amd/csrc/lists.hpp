@@ -1149,6 +1149,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
     static const int tune_wpb = getenv("SPTMM_WAVES_PER_WG") ? atoi(getenv("SPTMM_WAVES_PER_WG")) : 0;
     static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
+    static const int tune_tpw = getenv("SPTMM_TASKS_PER_WAVE") ? atoi(getenv("SPTMM_TASKS_PER_WAVE")) : 0;
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(lists_tile_rows(a) + 64) * SLOT;
     // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better
@@ -1203,6 +1204,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // four fp16 rows (sums on the matrix unit, 56 KB tile at K=6912), batched: eight wavefronts as well
     // (headline shape, 5 -> 8: u16 lists 69 -> 81 % of HBM peak, gap stream 39 -> 53 %)
     if (MT == 4 && sizeof(Act) == 2 && a.batch >= 4 && a.W == 1 && max_waves >= 8) wpb = 8;
+    // four fp32 rows (16-byte slots like eight int8 rows, sums on the VALU), batched: the largest workgroup, and tasks per
+    // wavefront by the search below (headline shape, 32 GEMVs: 5 wavefronts x 2 tasks 6.75 us per GEMV, 8 x 4 4.10,
+    // 8 x 10 -- two full rounds -- 3.73 us = 71 % of HBM peak; gap stream 4.13 -> 3.46 us)
+    if (MT == 4 && sizeof(Act) == 4 && a.batch >= 4 && a.W == 1) wpb = max_waves;
     if (tune_wpb > 0 && tune_wpb <= (a.quant ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>()) && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
@@ -1211,7 +1216,8 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // A batched launch has workgroups enough to fill the chip along blockIdx.z, and every workgroup
     // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
     // per GEMV, four-row tiles 2.83 -> 2.76; nothing for the one-row u16 kernel, which waits on HBM only).
-    if ((MT == 8 || (MT == 4 && MODE != 0)) && a.batch >= 4 && wgs == 1) {
+    constexpr bool WIDE_SLOT = MT == 8 || (MT == 4 && sizeof(Act) == 4);  // 16 bytes per index
+    if ((WIDE_SLOT || (MT == 4 && MODE != 0)) && a.batch >= 4 && wgs == 1) {
         // Multi-row tiles are expensive to stage (eight rows of K=13824: 110 KB, ~2.5 us against ~4 us per task) and their
         // walks are bound by the LDS and the matrix unit rather than by HBM: up to 16 tasks per wavefront, chosen so that the
         // launch's workgroups come in full rounds over the workgroups the chip holds at once (cost per round: staging
@@ -1220,13 +1226,13 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         // (12 tasks -- one and a third rounds -- 18.9 us); 14 gap-stream GEMVs, 8 / 12 tasks 10.1 / 9.8 us (10 tasks: 2.35
         // rounds, 10.9 us); K=6912 N=2560 split_k=32, M=4, 32 gap-stream GEMVs, 2 / 5 / 10 tasks 2.18 / 2.01 / 1.94 us
         // (int8 rows), 2.50 / 2.19 / 2.05 us (fp16 rows); K=13824, four fp16 rows, 2 / 12 tasks 16.1 / 11.6 us.
-        // u16 lists on four-row tiles wait on HBM and gain nothing from more than two tasks.
+        // u16 lists on four-row tiles of int8 or fp16 rows wait on HBM and gain nothing from more than two tasks.
         const size_t per_wg = tile + lists_behind_tile<Act, MT>(wpb);
         const int by_lds = (int)((size_t)a.lds_limit / per_wg), by_regs = 4 * waves_per_simd / wpb;
         const int resident = std::max(1, std::min(by_lds, by_regs));
         const long at_once = (long)cus * resident;
         const int row_tiles = (a.M + MT - 1) / MT;
-        const double stage = MT == 8 ? 2.5 : 2.0, walk = MT == 8 ? 4.0 : 5.7;
+        const double stage = WIDE_SLOT ? 2.5 : 2.0, walk = WIDE_SLOT ? 4.0 : 5.7;
         double best = 1e30;
         int pick = iters;
         for (int t = 1; t <= 16 && t <= blocks; ++t) {
@@ -1239,6 +1245,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     } else if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && MT == 1)) {
         grid_x = (blocks + 1) / 2;
         iters = 2;
+    }
+    if (tune_tpw > 0 && a.batch) {
+        grid_x = (blocks + tune_tpw - 1) / tune_tpw;
+        iters = (blocks + grid_x - 1) / grid_x;
     }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
                  a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale, a.stones};
