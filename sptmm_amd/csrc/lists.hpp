@@ -1147,9 +1147,12 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // tiles take.  Measured on MI355X, K=2560 N=13824 split_k=32: one workgroup per CU 11.4 us,
     // two 6.3 us; the headline shape has 5 tasks per CU and stays at one workgroup of 5.
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
-    static const int tune_wpb = getenv("SPTMM_WAVES_PER_WG") ? atoi(getenv("SPTMM_WAVES_PER_WG")) : 0;
-    static const int tune_wgs = getenv("SPTMM_WGS_PER_CU") ? atoi(getenv("SPTMM_WGS_PER_CU")) : 0;
-    static const int tune_tpw = getenv("SPTMM_TASKS_PER_WAVE") ? atoi(getenv("SPTMM_TASKS_PER_WAVE")) : 0;
+    // launch-shape overrides for tuning runs; read once, or at every launch when SPTMM_TUNE_LIVE is set
+    auto knob = [](const char *name) { const char *v = getenv(name); return v ? atoi(v) : 0; };
+    static const bool tune_live = getenv("SPTMM_TUNE_LIVE") != nullptr;
+    static const int wpb0 = knob("SPTMM_WAVES_PER_WG"), wgs0 = knob("SPTMM_WGS_PER_CU"), tpw0 = knob("SPTMM_TASKS_PER_WAVE");
+    const int tune_wpb = tune_live ? knob("SPTMM_WAVES_PER_WG") : wpb0, tune_wgs = tune_live ? knob("SPTMM_WGS_PER_CU") : wgs0,
+              tune_tpw = tune_live ? knob("SPTMM_TASKS_PER_WAVE") : tpw0;
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(lists_tile_rows(a) + 64) * SLOT;
     // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better
@@ -1187,9 +1190,14 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             }
         }
     }
-    // byte rows, batched: the tile is a quarter of the others' and the chip is filled along blockIdx.z; the largest
-    // workgroup does best (headline shape, 32 GEMVs per launch: 5 wavefronts 77 %, 8 wavefronts 79 % of HBM peak)
-    if (is_byte_rows<Act>() && a.batch) wpb = max_waves / a.W * a.W;
+    // byte rows, batched: the tile is a quarter of the others' and the chip is filled along blockIdx.z; small workgroups
+    // of four wavefronts, many per CU, do best (32 GEMVs per launch, 8 -> 4 wavefronts: K=6912 N=2560 1.65 -> 1.54 us
+    // per GEMV, K=2560 N=2560 0.72 -> 0.65, K=13824 N=5120 6.8 -> 6.3; sparse streams with zero slots 0.36-0.86 ->
+    // 0.33-0.81 us)
+    if (is_byte_rows<Act>() && a.batch && a.W == 1) wpb = 4;
+    // u16 lists on one- and four-row int8 tiles, batched, more tasks than the headline shape's 1280: eight wavefronts
+    // (K=13824 N=5120: M=1 12.9 -> 12.3 us per GEMV, M=4 13.5 -> 12.6; K=2560 N=6912, M=4: 3.2 -> 3.0 us)
+    if (MODE == 0 && MT <= 4 && sizeof(Act) == 1 && !is_byte_rows<Act>() && a.batch >= 4 && a.W == 1 && a.tasks >= 1536 && max_waves >= 8) wpb = 8;
     // eight-row tiles keep the matrix unit busy: a batched launch takes a wavefront count the four SIMDs share evenly
     // (K=13824 N=5120, M=8, 10 -> 12 wavefronts: gap stream 48 -> 55 % of HBM peak, u16 lists level)
     // -- and the largest workgroup does best: four wavefronts per SIMD, fewer workgroups staging (same shape, 12 -> 16
@@ -1198,9 +1206,11 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // way, and one workgroup of 16 stages the tile once -- K=6912 N=2560, M=8, 8 -> 16 wavefronts: u16 3.65 -> 3.40 us, gap
     // stream level at 2.14-2.40 us from box to box)
     if (MT == 8 && a.batch >= 4 && a.W == 1 && !a.quant) wpb = lists_max_waves<Act, MT, false>() / 4 * 4;
-    // four-row tiles on gap streams, batched, tile small enough for several workgroups per CU: eight wavefronts
-    // (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824 five do better)
-    if (MT == 4 && MODE != 0 && a.batch >= 4 && a.W == 1 && tile <= 40 * 1024 && max_waves >= 8) wpb = 8;
+    // four-row tiles on gap streams, batched, tile small enough for several workgroups per CU: four wavefronts for
+    // int8 rows (K=2560 N=640 0.32 -> 0.29 us per GEMV, M=2 on the headline shape 1.76 -> 1.67; level elsewhere), eight
+    // for fp16 rows (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824
+    // five do better)
+    if (MT == 4 && MODE != 0 && a.batch >= 4 && a.W == 1 && tile <= 40 * 1024 && max_waves >= 8) wpb = sizeof(Act) == 1 ? 4 : 8;
     // four fp16 rows (sums on the matrix unit, 56 KB tile at K=6912), batched: eight wavefronts as well
     // (headline shape, 5 -> 8: u16 lists 69 -> 81 % of HBM peak, gap stream 39 -> 53 %)
     if (MT == 4 && sizeof(Act) == 2 && a.batch >= 4 && a.W == 1 && max_waves >= 8) wpb = 8;
@@ -1211,7 +1221,9 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     if (tune_wpb > 0 && tune_wpb <= (a.quant ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>()) && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
-    int grid_x = blocks < slots ? blocks : slots;
+    // one GEMV per launch: no more workgroups than the chip holds at once; a batched launch fills the chip along
+    // blockIdx.z and starts from one task per wavefront
+    int grid_x = a.batch >= 8 || blocks < slots ? blocks : slots;
     int iters = (blocks + grid_x - 1) / grid_x;
     // A batched launch has workgroups enough to fill the chip along blockIdx.z, and every workgroup
     // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
@@ -1237,12 +1249,20 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         int pick = iters;
         for (int t = 1; t <= 16 && t <= blocks; ++t) {
             const long total = (long)a.batch * row_tiles * ((blocks + t - 1) / t);
-            const double cost = (double)((total + at_once - 1) / at_once) * (stage + walk * t);
+            // Workgroups of four wavefronts on small tiles sit four or five to a CU and share its throughput: what counts is
+            // the number of workgroups per CU, each costing a quarter of a task's walk to stage (hidden behind the others)
+            // plus its tasks, and the last one's length (K=6912 N=2560, M=4, 32 GEMVs: 1 / 2 / 4 / 5 / 8 / 10 tasks 2.04 /
+            // 1.82 / 1.77 / 1.76 / 1.80 / 1.83 us; K=2560 N=6912: 2.15 / 1.86 / 1.85 / 1.89 / 1.92 / 2.10 us).
+            const double cost = MT == 4 && sizeof(Act) == 1 && wpb == 4 ? (double)((total + cus - 1) / cus) * (0.25 + t) + 0.5 * t
+                                                                         : (double)((total + at_once - 1) / at_once) * (stage + walk * t);
             if (cost < best - 1e-9) best = cost, pick = t;
         }
         grid_x = (blocks + pick - 1) / pick;
         iters = (blocks + grid_x - 1) / grid_x;
-    } else if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && MT == 1)) {
+    } else if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && (MT == 1 || (MT == 4 && sizeof(Act) == 1))) &&
+               !(is_byte_rows<Act>() && !VAR && task_kb >= 8.0 && tile <= (size_t)(task_kb * 1024.0))) {
+        // (byte rows whose task is 8 KB or more and no smaller than the tile: one task per wavefront, 1.54 against 1.63 us
+        // on the headline shape; shorter tasks and larger tiles do better with two)
         grid_x = (blocks + 1) / 2;
         iters = 2;
     }
