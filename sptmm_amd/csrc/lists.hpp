@@ -69,21 +69,22 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
     static constexpr int SLOT = slot_bytes<Act, MT>();
     static_assert(!PLAIN || sizeof(Act) == 2, "only fp16 tiles have a VALU twin");
     static constexpr bool MX = sizeof(Act) == 1 && MT > 1;  // sums on the matrix unit
-    static constexpr bool MXF = sizeof(Act) == 2 && MT > 1 && !PLAIN;  // the same for fp16 rows (MT = 4): v_mfma_f32_16x16x32_f16,
-                                                                       // two entries x four rows per operand, selector of 0 / +-1.0
+    static constexpr bool MXF = sizeof(Act) == 2 && MT > 1 && !PLAIN;  // the same for fp16 rows: v_mfma_f32_16x16x32_f16, two entries x
+                                                                       // four rows (MT = 4) or one entry x eight rows (MT = 8) per
+                                                                       // operand, selector of 0 / +-1.0
     static constexpr int NW = MX ? MT / 4 : 1;              // dwords per gathered slot (int8)
-    static constexpr int ND = MX ? MT / 4 : 1;              // result tiles
+    static constexpr int ND = (MX || MXF) ? MT / 4 : 1;     // result tiles
     v4i D[ND], Bp[ND], Bn[ND];                              // MX: 16x16 int32 result tiles and the +1 / -1 selectors
     bool merged = false;                                    // MT = 8, columns of 32 or 64 lanes: one result tile sums lanes i, i+16 (, i+32, i+48)
-    v4f Df;                                                 // MXF: the fp32 result tile ...
-    v8h Bpf, Bnf;                                           // ... and its selectors
+    v4f Df[ND];                                             // MXF: the fp32 result tiles ...
+    v8h Bpf[ND], Bnf[ND];                                   // ... and their selectors
     A acc[MT];
 
     // sum of the four registers a lane holds of result tile x
     __device__ __forceinline__ A tile_sum(int x) const
     {
         if constexpr (MXF)
-            return (Df[0] + Df[1]) + (Df[2] + Df[3]);
+            return (Df[x][0] + Df[x][1]) + (Df[x][2] + Df[x][3]);
         else
             return (A)(D[x][0] + D[x][1] + D[x][2] + D[x][3]);
     }
@@ -119,14 +120,24 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                 D[x] = v4i{0, 0, 0, 0};
             }
         } else if constexpr (MXF) {
+            // lane j + 16 g holds rows 8 g .. 8 g + 7 of selector column j.  MT = 4: the operand is two entries x four
+            // rows, column 4 g + row.  MT = 8: one entry x eight rows; tiles and columns as for eight int8 rows.
+            merged = MT == 8 && logL >= 5;
             const int l = threadIdx.x & 63, g = l >> 4, j = l & 15;
 #pragma unroll
-            for (int y = 0; y < 8; ++y) {
-                const bool on = (j >> 2) == g && (y & 3) == (j & 3);
-                Bpf[y] = on ? (_Float16)1.0f : (_Float16)0.0f;
-                Bnf[y] = on ? (_Float16)-1.0f : (_Float16)0.0f;
+            for (int x = 0; x < ND; ++x) {
+#pragma unroll
+                for (int y = 0; y < 8; ++y) {
+                    bool on;
+                    if constexpr (MT == 4)
+                        on = (j >> 2) == g && (y & 3) == (j & 3);
+                    else
+                        on = (merged ? (x == 0 && (j >> 3) == (logL == 5 ? g >> 1 : 0)) : ((g >> 1) == x && (j >> 3) == (g & 1))) && y == (j & 7);
+                    Bpf[x][y] = on ? (_Float16)1.0f : (_Float16)0.0f;
+                    Bnf[x][y] = on ? (_Float16)-1.0f : (_Float16)0.0f;
+                }
+                Df[x] = v4f{0.f, 0.f, 0.f, 0.f};
             }
-            Df = v4f{0.f, 0.f, 0.f, 0.f};
         }
     }
 
@@ -156,6 +167,15 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                     if (!merged) D[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[1] : Bp[1], D[1], 0, 0, 0);  // (uniform)
                 }
             }
+        } else if constexpr (MXF && MT == 8) {
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                v8h a;
+#pragma unroll
+                for (int m = 0; m < 8; ++m) a[m] = r[e].v[m];
+                Df[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[0] : Bpf[0], Df[0], 0, 0, 0);
+                if (!merged) Df[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[1] : Bpf[1], Df[1], 0, 0, 0);  // (uniform)
+            }
         } else if constexpr (MXF) {
 #pragma unroll
             for (int e = 0; e < NE; e += 2) {
@@ -165,7 +185,7 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                     a[m] = r[e].v[m];
                     a[4 + m] = e + 1 < NE ? r[e + 1 < NE ? e + 1 : e].v[m] : (_Float16)0.0f;
                 }
-                Df = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf : Bpf, Df, 0, 0, 0);
+                Df[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[0] : Bpf[0], Df[0], 0, 0, 0);
             }
         } else {
 #pragma unroll
@@ -441,6 +461,17 @@ template <typename Act, int MT> struct Stager {
             for (int j = 0; j < 4; ++j) {
                 u32 d0 = comp(r[j / 2], (2 * j) % 4), d1 = comp(r[j / 2], (2 * j + 1) % 4);
                 t[4 * item + j] = make_uint4(f2u(h2f(d0, 0)), f2u(h2f(d0, 1)), f2u(h2f(d1, 0)), f2u(h2f(d1, 1)));
+            }
+        } else if constexpr (sizeof(Act) == 2 && MT == 8) {  // [k][8 halves]; r[2m+h] = row m, halves 8h..8h+7
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {  // k = 16*item + 2i, 2i+1
+                u32 d[8];
+#pragma unroll
+                for (int m = 0; m < 8; ++m) d[m] = comp(r[2 * m + i / 4], i % 4);
+                t[16 * item + 2 * i] = make_uint4((d[0] & 0xffffu) | (d[1] << 16), (d[2] & 0xffffu) | (d[3] << 16),
+                                                  (d[4] & 0xffffu) | (d[5] << 16), (d[6] & 0xffffu) | (d[7] << 16));
+                t[16 * item + 2 * i + 1] = make_uint4((d[0] >> 16) | (d[1] & 0xffff0000u), (d[2] >> 16) | (d[3] & 0xffff0000u),
+                                                      (d[4] >> 16) | (d[5] & 0xffff0000u), (d[6] >> 16) | (d[7] & 0xffff0000u));
             }
         } else if constexpr (sizeof(Act) == 2) {  // MT == 4: [k][4 halves]; r[2m+h] = row m, halves 8h..8h+7
 #pragma unroll
@@ -995,7 +1026,7 @@ struct ListsBody {
                 const int logL = p.logL;
                 A t[ND];
                 bool merged_done = false;
-                if constexpr (Sums<Act, MT>::MX && MT == 8) {
+                if constexpr (MT == 8) {
                     if (acc.merged) {
                         // one tile: lane l, register r = rows i = 4 (l >> 4) + r, result column j = l & 15 holds activation
                         // row j & 7 of the task's column j >> 3; the 16 i are the column's lanes i, i+16 (, i+32, i+48)
@@ -1364,7 +1395,7 @@ static int launch_lists_m(const GemvArgs &a, hipStream_t st)
         const size_t extra = a.quant ? (size_t)(2 * LISTS_MAX_WAVES + 1) * mt * 4 : behind;
         return (size_t)(lists_tile_rows(a) + 64) * slot + extra <= (size_t)a.lds_limit;
     };
-    if constexpr (sizeof(Act) == 1) {
+    if constexpr (sizeof(Act) <= 2) {  // int8 and fp16 rows; four fp32 rows already fill a 16-byte slot
         if (a.M >= 5 && fits(slot_bytes<Act, 8>(), 8, lists_behind_tile<Act, 8>(lists_max_waves<Act, 8, false>())))
             return launch_lists_t<Act, 8, MODE, PRE, VAR>(a, st);
     }

@@ -292,6 +292,24 @@ def test_u16_float_activations(dtype, M):
         check_fp(got, ref, S)
 
 
+@pytest.mark.parametrize("K,N,S", [(6912, 2560, 4096), (2560, 640, 1536)])
+@pytest.mark.parametrize("M", [5, 8, 9, 16])
+def test_fp16_eight_row_tiles(K, N, S, M):
+    """Five to eight fp16 rows share one tile of 16-byte slots (all eight rows of an index) and are summed on the matrix
+    unit; every lanes-per-column case of its result layout (8, 16, 32, 64 lanes, and columns that span wavefronts), on
+    u16 lists and on gap streams, against the fp64 oracle to the usual 1e-3."""
+    _, pos, neg = matrix(K, N, S)
+    X = oracle.make_x_normal(70 + M, M, K, np.float16)
+    ref = oracle.sptmm_f64(X, pos, neg)
+    for kind, splits in (("u16", (8, 16, 32, 64, 128)), ("delta", (8, 16, 32, 64))):
+        for split in splits:
+            say("fp16 eight rows", K, N, S, "M", M, kind, split)
+            w = sp.Weights.upload_u16(pos, neg, K, split) if kind == "u16" else sp.Weights.upload_delta(pos, neg, K, split)
+            got = w.matmul(X)
+            w.free()
+            check_fp(got, ref, S)
+
+
 def finite_columns(pos, neg, k):
     """Columns whose lists do not hold row k."""
     return ~((pos == k).any(axis=1) | (neg == k).any(axis=1))
@@ -306,7 +324,7 @@ def test_non_finite_activation_stays_in_its_row_and_columns(kind, split, bad):
     K, N, S = 2560, 640, 1536
     _, pos, neg = matrix(K, N, S)
     w = sp.Weights.upload_u16(pos, neg, K, split) if kind == "u16" else sp.Weights.upload_delta(pos, neg, K, split)
-    for M, dtype in ((4, np.float16), (3, np.float16), (1, np.float16), (4, np.float32)):
+    for M, dtype in ((4, np.float16), (3, np.float16), (1, np.float16), (4, np.float32), (8, np.float16), (6, np.float16)):
         for k in (0, 1337, K - 1):
             say("non-finite", kind, split, dtype.__name__, "M", M, "k", k, bad)
             X = oracle.make_x_normal(500 + M + k, M, K, dtype)
