@@ -516,7 +516,15 @@ constexpr int LISTS_MAX_WAVES = 8;  // 512 threads: two wavefronts per SIMD, 256
 // Multi-row int8 tiles do several times the arithmetic per stream byte, and a large K leaves
 // room for one workgroup per CU only, so that workgroup has to bring the wavefronts that fill
 // the four SIMDs itself: 1024 threads, four wavefronts per SIMD, 128 VGPRs each.
-template <typename Act, int MT, bool QUANT> constexpr int lists_max_waves() { return sizeof(Act) == 1 && MT >= 4 && !QUANT ? 16 : LISTS_MAX_WAVES; }
+// The same for four fp32 rows (16-byte slots, a tile as large as eight int8 rows' twice over: headline shape, M=4, 32 GEMVs
+// per launch, 8 -> 16 wavefronts: u16 3.66 -> 3.58 us per GEMV, gap stream 3.48 -> 3.26).  Eight fp16 rows stay at 512
+// threads: their gathers of 16 entries x 16 bytes do not fit 128 registers (up to 272 bytes of scratch per lane).
+// Kernels that run at 128 registers keep a ring of four rounds and no straight-line body beyond four.
+template <typename Act, int MT> constexpr bool lists_short_of_registers() { return (MT == 8 && sizeof(Act) == 1) || (MT == 4 && sizeof(Act) == 4); }
+template <typename Act, int MT, bool QUANT> constexpr int lists_max_waves()
+{
+    return ((sizeof(Act) == 1 && MT >= 4) || lists_short_of_registers<Act, MT>()) && !QUANT ? 16 : LISTS_MAX_WAVES;
+}
 
 // LDS a workgroup of `waves` wavefronts keeps behind the activation tile: the per-wavefront sums of
 // columns that span wavefronts, and for fp16 tiles summed on the matrix unit one flag per wavefront.
@@ -614,7 +622,7 @@ struct ListsBody {
     static constexpr int ZROWS = 64;                  // zero slots behind the tile (row K, and the padding rows)
     static constexpr int SH = ilog2(SLOT_OF);
     static constexpr int SLOT = SLOT_OF;
-    static constexpr int RING = MT == 8 ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
+    static constexpr int RING = lists_short_of_registers<Act, MT>() ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
     static constexpr int XMAX = VAR ? 2 : 0;          // ragged tasks on the straight-line path: full rounds beyond RF a task may have
     static constexpr int EARLY = MT >= 4 ? 4 : 2;     // rounds requested before the activation tile is complete (multi-row tiles take longer to stage)
 
@@ -1365,7 +1373,7 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
         }
         // Eight-row kernels are short of registers (1024-thread workgroups, 128 VGPRs): beyond four rounds the
         // ring of four does better than a straight-line body that holds six or eight (K=13824 M=8: 15.4 -> 14.4 us).
-        if (MT == 8 && rf > 4) rf = 9;  // no straight-line body of that length: falls through to the ring
+        if (lists_short_of_registers<Act, MT>() && rf > 4) rf = 9;  // no straight-line body of that length: falls through to the ring
         switch (rf) {
         case 0:
             if ((VAR ? a.n_max : a.n_lane) / E16 <= ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) return launch_lists_rf<Act, MT, MODE, PRE, VAR, -1>(a, st);
@@ -1375,10 +1383,10 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
         case 3: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 3>(a, st);
         case 4: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 4>(a, st);
         case 6:
-            if constexpr (MT != 8) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 6>(a, st);
+            if constexpr (!lists_short_of_registers<Act, MT>()) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 6>(a, st);
             break;
         case 8:
-            if constexpr (MT != 8) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 8>(a, st);
+            if constexpr (!lists_short_of_registers<Act, MT>()) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 8>(a, st);
             break;
         default: break;
         }
