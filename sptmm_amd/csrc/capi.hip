@@ -157,6 +157,21 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
         if (quant) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
         return launch_wide(a, w->wh, act, stream);
     }
+    // A ragged stream whose tasks all hold the same number of entries, and whose tile keeps no zero slots, is laid out
+    // behind its count table exactly like a stream of balanced lists (the packers share slot_offset()): it runs on the
+    // kernels for tasks of one length -- no table look-ups, straight-line bodies of the exact length (K=6912 N=2560, 864
+    // entries per list, 32 GEMVs per launch: 0.81 -> 0.75 us per GEMV).
+    std::vector<const void *> behind_table;
+    if (a.ragged && a.n_min == a.n_max && !a.stones && w->info.kind != SPTMM_KIND_I2S) {
+        a.ragged = 0;
+        a.n_lane = a.n_max;
+        a.w = (const uint8_t *)w->dev + w->counts_bytes;
+        if (batch) {
+            behind_table.resize(batch);
+            for (int i = 0; i < batch; ++i) behind_table[i] = (const uint8_t *)bw[i] + w->counts_bytes;
+            a.batch_w = behind_table.data();
+        }
+    }
     switch (w->info.kind) {
     case SPTMM_KIND_U16: return launch_u16(a, act, stream);
     case SPTMM_KIND_DELTA: return launch_delta(a, act, stream);

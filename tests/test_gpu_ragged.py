@@ -165,3 +165,34 @@ def test_outputs_match_golden_fixture(golden_dir):
             w.free()
             assert got[0, :8].tolist() == e["C_head"]
             assert hashlib.sha256(got.tobytes()).hexdigest() == e["sha256_C"]
+
+
+@pytest.mark.parametrize("K,N,S,split", [(6912, 2560, 1728, 16), (2560, 640, 1536, 32), (2560, 640, 1536, 8)])
+def test_ragged_stream_with_tasks_of_one_length(K, N, S, split):
+    """A balanced matrix packed from its dense form is a ragged stream whose tasks all have one length; behind its count
+    table it is laid out like the stream of balanced lists, and the launch takes the kernels for tasks of one length.
+    Same results as the balanced stream and the oracle: u16 lists, gap streams for four-byte and one-byte rows, one
+    row, a four-row and an eight-row tile, alone and in a batched launch."""
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    for M in (1, 4, 8):
+        X = oracle.make_x_i8(30 + M, M, K)
+        ref = oracle.sptmm_i8_mt(X, pos, neg, 8)
+        for kind, rows in ((sp.KIND_U16, 0), (sp.KIND_DELTA, 0), (sp.KIND_DELTA, 1)):
+            say("uniform ragged", K, N, S, split, "M", M, "kind", kind, "rows", rows)
+            w = sp.Weights.upload_dense(W, kind, split, rows=rows)
+            assert w.info["ragged"] == 1 and w.info["stones"] == 0
+            assert np.array_equal(w.matmul(X), ref)
+            xb = [sp.DeviceBuffer.from_numpy(X) for _ in range(8)]
+            cb = [sp.DeviceBuffer(4 * M * N) for _ in range(8)]
+            sp.gemv_batched([w] * 8, xb, cb, M, 0)
+            sp.device_sync()
+            for c in cb:
+                assert np.array_equal(c.to_numpy(np.int32, (M, N)), ref)
+            for o in [w] + xb + cb:
+                o.free()
+    Xh = oracle.make_x_normal(77, 4, K, np.float16)
+    w = sp.Weights.upload_dense(W, sp.KIND_DELTA, split)
+    got = w.matmul(Xh)
+    w.free()
+    ref = oracle.sptmm_f64(Xh, pos, neg)
+    assert np.abs(got - ref).max() <= 1e-3 * max(1.0, np.abs(ref).max())
