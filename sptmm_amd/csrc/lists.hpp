@@ -164,7 +164,9 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                             e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[1] : 0};
                 D[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[0] : Bp[0], D[0], 0, 0, 0);
                 if constexpr (ND > 1) {
-                    if (!merged) D[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[1] : Bp[1], D[1], 0, 0, 0);  // (uniform)
+                    // (uniform.  A loop of its own for the second tile, one branch per call instead of one per instruction,
+                    // keeps the operands alive across both loops and was slower: K=6912 N=2560, gap stream, M=8 2.0 -> 2.4 us)
+                    if (!merged) D[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[1] : Bp[1], D[1], 0, 0, 0);
                 }
             }
         } else if constexpr (MXF && MT == 8) {
@@ -174,7 +176,15 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
 #pragma unroll
                 for (int m = 0; m < 8; ++m) a[m] = r[e].v[m];
                 Df[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[0] : Bpf[0], Df[0], 0, 0, 0);
-                if (!merged) Df[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[1] : Bpf[1], Df[1], 0, 0, 0);  // (uniform)
+            }
+            if (!merged) {  // (uniform; a loop of its own: one branch per call)
+#pragma unroll
+                for (int e = 0; e < NE; ++e) {
+                    v8h a;
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) a[m] = r[e].v[m];
+                    Df[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[1] : Bpf[1], Df[1], 0, 0, 0);
+                }
             }
         } else if constexpr (MXF) {
 #pragma unroll
