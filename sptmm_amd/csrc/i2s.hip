@@ -18,6 +18,7 @@ struct I2sParams {
     const int8_t *X;
     int *C;
     int M, K, Kp, N, rounds;
+    int threads;  // blockDim.x as an argument (the built-in costs two memory round trips in a row at kernel start)
 };
 
 // Workgroup = 16 columns; wavefront `wave` takes rounds wave, wave+waves, ...;
@@ -29,9 +30,9 @@ __device__ __forceinline__ void i2s_body(const I2sParams &p, unsigned char *smem
 {
     int8_t *lx = reinterpret_cast<int8_t *>(smem);                       // [MT][Kp]
     int *part = reinterpret_cast<int *>(smem + (size_t)MT * p.Kp);      // [waves][16][MT]
-    int *sums = part + (blockDim.x >> 6) * 16 * MT;                      // [waves][MT]
+    int *sums = part + (p.threads >> 6) * 16 * MT;                      // [waves][MT]
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = p.threads >> 6;
     const int grp = blockIdx.x, m0 = blockIdx.y * MT;
     constexpr int RPB = 4;
 
@@ -49,7 +50,7 @@ __device__ __forceinline__ void i2s_body(const I2sParams &p, unsigned char *smem
         rs[m] = 0;
         const uint4 *src = reinterpret_cast<const uint4 *>(p.X + (size_t)(m0 + m) * p.K);
         uint4 *dst = reinterpret_cast<uint4 *>(lx + (size_t)m * p.Kp);
-        for (int i = tid; i < p.Kp / 16; i += blockDim.x) {
+        for (int i = tid; i < p.Kp / 16; i += p.threads) {
             uint4 v = make_uint4(0, 0, 0, 0);
             if (m0 + m < p.M && i < p.K / 16) v = src[i];
             dst[i] = v;
@@ -104,7 +105,7 @@ __device__ __forceinline__ void i2s_body(const I2sParams &p, unsigned char *smem
         if (q == 0) part[(wave * 16 + lane) * MT + m] = acc[m];
     }
     __syncthreads();
-    for (int t = tid; t < 16 * MT; t += blockDim.x) {
+    for (int t = tid; t < 16 * MT; t += p.threads) {
         const int col = t / MT, m = t % MT;
         int s = 0, sx = 0;
         for (int w = 0; w < waves; ++w) {
@@ -216,7 +217,7 @@ __device__ __forceinline__ void i2s_mfma_round(const I2sRound<XJ, CT> &o, unsign
 template <int XJ, int CT>
 __device__ __forceinline__ void i2s_mfma_body(const I2sParams &p, unsigned char *smem)
 {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = p.threads >> 6;
     const int m0 = blockIdx.y * 16, groups = p.N / 16;
     unsigned char *patch = smem + (size_t)wave * (CT > 4 ? CT : 4) * 1024;  // this wavefront's 16 rows x 256 k (and its sums at the end)
     const int8_t *xrow[XJ];
@@ -265,7 +266,7 @@ __device__ __forceinline__ void i2s_mfma_body(const I2sParams &p, unsigned char 
 #pragma unroll
         for (int r = 0; r < 4; ++r) part[c * 256 + (4 * (lane >> 4) + r) * 16 + (lane & 15)] = D[c][r] - 2 * D1[r];
     __syncthreads();
-    for (int t = tid; t < 256 * CT; t += blockDim.x) {
+    for (int t = tid; t < 256 * CT; t += p.threads) {
         int s = 0;
         for (int w = 0; w < waves; ++w) s += reinterpret_cast<const int *>(smem + (size_t)w * (CT > 4 ? CT : 4) * 1024)[t];
         const int m = m0 + ((t & 255) >> 4), g = blockIdx.x * CT + (t >> 8);
@@ -298,11 +299,12 @@ __global__ void __launch_bounds__(256) copy_kernel(uint4 *dst, const uint4 *src,
 // Streaming read of a buffer with the list kernels' own load instruction (16 bytes per lane,
 // non-temporal), every lane folding what it reads into one word that is written at the end:
 // the ceiling the GEMV kernels can be held against.
-__global__ void __launch_bounds__(512) read_kernel(const v4u *src, size_t n16, u32 *sink)
+// (`threads`: every thread of the launch, as an argument like the GEMV kernels' block and grid sizes.)
+__global__ void __launch_bounds__(512) read_kernel(const v4u *src, size_t n16, u32 *sink, size_t threads)
 {
     v4u a = {0, 0, 0, 0};
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = threads;
+    size_t i = (size_t)blockIdx.x * 512 + threadIdx.x;
     for (; i + 3 * stride < n16; i += 4 * stride) {
         v4u x0 = __builtin_nontemporal_load(src + i), x1 = __builtin_nontemporal_load(src + i + stride);
         v4u x2 = __builtin_nontemporal_load(src + i + 2 * stride), x3 = __builtin_nontemporal_load(src + i + 3 * stride);
@@ -333,7 +335,7 @@ template <int MT>
 static int launch_i2s_t(const GemvArgs &a, hipStream_t st, int waves)
 {
     const int Kp = i2s_padded_k(a.K);
-    I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256};
+    I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256, 64 * waves};
     size_t lds = (size_t)MT * Kp + (size_t)waves * 16 * MT * 4 + (size_t)waves * MT * 4;
     dim3 grid(a.N / 16, (a.M + MT - 1) / MT), block(64 * waves);
     if (a.batch) {
@@ -367,7 +369,7 @@ template <int XJ, int CT>
 static int launch_i2s_mfma_t(const GemvArgs &a, hipStream_t st, int waves)
 {
     const int Kp = i2s_padded_k(a.K), groups = a.N / 16;
-    I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256};
+    I2sParams p{(const uint4 *)a.w, (const int8_t *)a.X, (int *)a.C, a.M, a.K, Kp, a.N, Kp / 256, 64 * waves};
     const size_t lds = (size_t)waves * (CT > 4 ? CT : 4) * 1024;
     dim3 grid((groups + CT - 1) / CT, (a.M + 15) / 16), block(64 * waves);
     static std::atomic<size_t> lds_granted{48 * 1024}, lds_granted_b{48 * 1024};
@@ -464,7 +466,8 @@ int launch_read(const void *src, size_t bytes, void *sink, int workgroups, void 
 {
     if (bytes % 16) return fail(SPTMM_ERR_INVALID, "read size must be a multiple of 16 bytes");
     if (workgroups < 1) workgroups = 256 * 4;
-    hipLaunchKernelGGL(read_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (const v4u *)src, bytes / 16, (u32 *)sink);
+    hipLaunchKernelGGL(read_kernel, dim3(workgroups), dim3(512), 0, (hipStream_t)stream, (const v4u *)src, bytes / 16, (u32 *)sink,
+                       (size_t)workgroups * 512);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "read_kernel launch");
 }

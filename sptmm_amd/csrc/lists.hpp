@@ -517,6 +517,10 @@ struct ListParams {
     int quant;      // quantising kernels: X holds 1 = fp16, 2 = bf16 values
     float w_scale;  // quantising kernels: factor applied to every output
     int stones;     // 8-bit gap streams of tile positions: the tile keeps 16 zero slots behind every 96 rows
+    // blockDim.x and gridDim.x, handed over as arguments: the built-ins are read from the dispatch's implicit arguments
+    // with a vector load whose address waits for a scalar load, two memory round trips in a row before the kernel's
+    // first activation or stream load is issued; these arrive with the other arguments in one
+    int threads, grid_x;
 };
 
 // rows of the activation tile in front of its 64 trailing zero rows
@@ -713,7 +717,7 @@ struct ListsBody {
         const int tile_rows = stones ? STONE_BLOCK * ((p.K + STONE_ROWS - 1) / STONE_ROWS) : p.K;
         auto place = [&](int item) { return stones ? item + item / (STONE_ROWS / 16) : item; };
         A *part = reinterpret_cast<A *>(smem + (size_t)(tile_rows + ZROWS) * SLOT);
-        const int tid = threadIdx.x, nt = blockDim.x;
+        const int tid = threadIdx.x, nt = p.threads;
         const int lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
         const int m0 = blockIdx.y * MT;
         const size_t task_bytes = VAR ? (size_t)p.task_stride : HDR + (size_t)128 * ESZ * p.n_lane;
@@ -722,7 +726,7 @@ struct ListsBody {
         // ragged: tasks differ in length; p.n_lane is the shortest, which is all the prologue may assume
         const int R0 = p.n_lane / E16;
         int task = blockIdx.x * waves + wave;
-        const int task_step = gridDim.x * waves;
+        const int task_step = p.grid_x * waves;
         const Act *X = reinterpret_cast<const Act *>(p.X);
         typedef Quantiser<MT> Q;
         const unsigned short *Xq = reinterpret_cast<const unsigned short *>(p.X);
@@ -1320,7 +1324,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         iters = (blocks + grid_x - 1) / grid_x;
     }
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, VAR ? a.n_min : a.n_lane, a.tasks, ilog2(a.L), a.W,
-                 a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale, a.stones};
+                 a.task_stride, a.counts_bytes, iters, a.quant, a.w_scale, a.stones, 64 * wpb, grid_x};
     size_t lds = tile + lists_behind_tile<Act, MT>(wpb);
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);

@@ -23,6 +23,7 @@ struct WideParams {
     const void *X;
     void *C;
     int M, K, N, k_tile, phases, tasks, logL, iters;
+    int threads, grid_x;  // blockDim.x and gridDim.x as arguments (the built-ins cost two memory round trips in a row at kernel start)
     u32 offset[16], stride[16];
     int n_min[16];
 };
@@ -275,7 +276,7 @@ template <typename Act, int MODE, int RING_ = 4> struct WideBody {
     // the parameter block itself untouched, so that it stays in scalar registers)
     static __device__ __forceinline__ void run(const WideParams &p, const uint8_t *w, const void *Xv, void *C, unsigned char *smem)
     {
-        const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
+        const int tid = threadIdx.x, nt = p.threads, lane = tid & 63, wave = tid >> 6, waves = nt >> 6;
         const int m0 = blockIdx.y * ROWS;
         const Act *X = reinterpret_cast<const Act *>(Xv);
         const int logL = p.logL, q = lane >> 4, row = lane & 15;
@@ -310,7 +311,7 @@ template <typename Act, int MODE, int RING_ = 4> struct WideBody {
             const unsigned short *counts = reinterpret_cast<const unsigned short *>(sub + RAGGED_PREAMBLE);
             const uint8_t *tasks_base = sub + ((size_t)16 + 2 * (size_t)p.tasks + 255) / 256 * 256;
             int task = blockIdx.x * waves + wave;
-            for (int it = 0; it < p.iters; ++it, task += gridDim.x * waves) {
+            for (int it = 0; it < p.iters; ++it, task += p.grid_x * waves) {
                 if (task >= p.tasks) break;  // (uniform per wavefront; no barrier inside the loop)
                 const int n = __builtin_amdgcn_readfirstlane((int)counts[task]);
                 const uint8_t *tb = tasks_base + (size_t)task * p.stride[ph];
@@ -413,6 +414,7 @@ static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
     p.w = (const uint8_t *)a.w, p.X = a.X, p.C = a.C;
     p.M = a.M, p.K = a.K, p.N = a.N, p.k_tile = h.k_tile, p.phases = h.phases, p.tasks = a.tasks, p.logL = ilog2(a.L);
     p.iters = (blocks + grid_x - 1) / grid_x;
+    p.threads = 64 * wpb, p.grid_x = grid_x;
     for (int i = 0; i < h.phases; ++i) p.offset[i] = h.offset[i], p.stride[i] = h.stride[i], p.n_min[i] = h.n_min[i];
     dim3 grid(grid_x, (a.M + ROWS - 1) / ROWS), block(64 * wpb);
     static std::atomic<size_t> lds_granted{48 * 1024}, lds_granted_b{48 * 1024};
