@@ -636,7 +636,10 @@ struct ListsBody {
     static constexpr int ZROWS = 64;                  // zero slots behind the tile (row K, and the padding rows)
     static constexpr int SH = ilog2(SLOT_OF);
     static constexpr int SLOT = SLOT_OF;
-    static constexpr int RING = lists_short_of_registers<Act, MT>() ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
+    // (four int8 rows also run 16 wavefronts per workgroup at 128 registers: their ragged kernels and the ones on 16-bit gaps
+    // keep the ring of four as well -- with eight they spilled 170-180 bytes per lane)
+    static constexpr bool TIGHT = lists_short_of_registers<Act, MT>() || (sizeof(Act) == 1 && !is_byte_rows<Act>() && MT == 4 && (VAR || Fl::GAP16));
+    static constexpr int RING = TIGHT ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
     static constexpr int XMAX = VAR ? 2 : 0;          // ragged tasks on the straight-line path: full rounds beyond RF a task may have
     static constexpr int EARLY = MT >= 4 ? 4 : 2;     // rounds requested before the activation tile is complete (multi-row tiles take longer to stage)
 
@@ -1387,7 +1390,9 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
         }
         // Eight-row kernels are short of registers (1024-thread workgroups, 128 VGPRs): beyond four rounds the
         // ring of four does better than a straight-line body that holds six or eight (K=13824 M=8: 15.4 -> 14.4 us).
-        if (lists_short_of_registers<Act, MT>() && rf > 4) rf = 9;  // no straight-line body of that length: falls through to the ring
+        if (lists_short_of_registers<Act, MT>() && rf > 4) rf = 9;
+        // four int8 rows on 16-bit gaps: straight-line bodies of four rounds and more spill (96-508 bytes per lane at 128 registers)
+        if (sizeof(Act) == 1 && MT == 4 && MODE == 2 && rf > 3) rf = 9;  // no straight-line body of that length: falls through to the ring
         switch (rf) {
         case 0:
             if ((VAR ? a.n_max : a.n_lane) / E16 <= ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) return launch_lists_rf<Act, MT, MODE, PRE, VAR, -1>(a, st);

@@ -449,8 +449,10 @@ static int launch_wide_t(const GemvArgs &a, const WideHeader &h, hipStream_t st)
     // fp16 rows on 8-bit gaps: 16 gathered slots of 16 bytes per stream dword do not fit 128 registers (152 bytes of scratch
     // per lane at 16 wavefronts); 12 wavefronts, 168 registers: K=13824 N=5120, M=8, one GEMV per launch 26.1 -> 22.2 us,
     // batched launches level (13.2 against 13.3 us)
-    if constexpr (sizeof(Act) == 2 && MODE == 1) return launch_wide_v<Act, MODE, 4, 12>(a, h, st);
-    return launch_wide_v<Act, MODE, 4, 16>(a, h, st);
+    if constexpr (sizeof(Act) == 2 && MODE == 1)
+        return launch_wide_v<Act, MODE, 4, 12>(a, h, st);
+    else
+        return launch_wide_v<Act, MODE, 4, 16>(a, h, st);
 }
 
 int launch_wide(const GemvArgs &a, const WideHeader &h, ActType act, void *stream)
