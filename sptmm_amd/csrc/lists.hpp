@@ -639,8 +639,8 @@ struct ListsBody {
     // (four int8 rows also run 16 wavefronts per workgroup at 128 registers: their ragged kernels and the ones on 16-bit gaps
     // keep the ring of four as well -- with eight they spilled 170-180 bytes per lane)
     static constexpr bool TIGHT = lists_short_of_registers<Act, MT>() || (sizeof(Act) == 1 && !is_byte_rows<Act>() && MT == 4 && (VAR || Fl::GAP16));
+    static constexpr int XMAX = VAR ? (TIGHT ? 1 : 2) : 0;  // ragged tasks on the straight-line path: full rounds beyond RF a task may have
     static constexpr int RING = TIGHT ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
-    static constexpr int XMAX = VAR ? 2 : 0;          // ragged tasks on the straight-line path: full rounds beyond RF a task may have
     static constexpr int EARLY = MT >= 4 ? 4 : 2;     // rounds requested before the activation tile is complete (multi-row tiles take longer to stage)
 
     static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, Sums<Act, MT> &acc)
