@@ -1392,7 +1392,8 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
         // ring of four does better than a straight-line body that holds six or eight (K=13824 M=8: 15.4 -> 14.4 us).
         if (lists_short_of_registers<Act, MT>() && rf > 4) rf = 9;
         // four int8 rows on 16-bit gaps: straight-line bodies of four rounds and more spill (96-508 bytes per lane at 128 registers)
-        if (sizeof(Act) == 1 && MT == 4 && MODE == 2 && rf > 3) rf = 9;  // no straight-line body of that length: falls through to the ring
+        constexpr bool UP_TO_THREE = sizeof(Act) == 1 && MT == 4 && MODE == 2;
+        if (UP_TO_THREE && rf > 3) rf = 9;  // no straight-line body of that length: falls through to the ring
         switch (rf) {
         case 0:
             if ((VAR ? a.n_max : a.n_lane) / E16 <= ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) return launch_lists_rf<Act, MT, MODE, PRE, VAR, -1>(a, st);
@@ -1400,12 +1401,14 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
         case 1: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 1>(a, st);
         case 2: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 2>(a, st);
         case 3: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 3>(a, st);
-        case 4: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 4>(a, st);
+        case 4:
+            if constexpr (!UP_TO_THREE) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 4>(a, st);
+            break;
         case 6:
-            if constexpr (!lists_short_of_registers<Act, MT>()) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 6>(a, st);
+            if constexpr (!lists_short_of_registers<Act, MT>() && !UP_TO_THREE) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 6>(a, st);
             break;
         case 8:
-            if constexpr (!lists_short_of_registers<Act, MT>()) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 8>(a, st);
+            if constexpr (!lists_short_of_registers<Act, MT>() && !UP_TO_THREE) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 8>(a, st);
             break;
         default: break;
         }
