@@ -240,6 +240,17 @@ def main():
             # (best of three: here the host has to issue a launch every 0.8 us, and anything else running on it shows)
             "cold_four_streams_us": round(min(timed(copies, n1, 256, 4)[0] for _ in range(3)), 3),
         }
+        # the same matrix at split-K 64 (one column per wavefront, ten wavefronts per CU instead of five): shorter wavefronts
+        # leave less gathering to do once the last bytes have arrived -- the library's faster shape for a lone launch
+        # (not BASELINE's configuration, which names split-K 32; slower than it in batched launches)
+        w64 = sp.Weights.upload_u16(pos, neg, K, 64)
+        assert (w64.matmul(X) == ref).all()
+        c64 = [w64] + [w64.clone() for _ in range(BATCH - 1)]
+        single["split64_cold_us"] = round(timed(c64, n1, 256, 0)[0], 3)
+        single["split64_warm_us"] = round(timed(c64[:1], n1, 256, 0)[0], 3)
+        single["split64_cold_pct_roofline"] = pct(nbytes, single["split64_cold_us"])
+        for c in c64:
+            c.free()
         single["cold_gbps"] = round(nbytes / single["cold_us"] / 1e3, 1)
         single["warm_gbps"] = round(nbytes / single["warm_us"] / 1e3, 1)
         single["cold_pct_roofline"] = pct(nbytes, single["cold_us"])
