@@ -62,7 +62,9 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 // row).  The matrix-unit sums multiply every byte of an operand row with 0 or +-1, so one Inf or
 // NaN among the gathered values turns the sums of the other rows and of the three partner lanes
 // into NaN (0 x Inf); a workgroup whose tile holds a non-finite value therefore sums this way.
-template <typename Act, int MT, bool PLAIN = false> struct Sums {
+// MERGED (eight-row tiles whose columns take 32 or 64 lanes, a property of the launch): one result tile where two are
+// needed otherwise -- half the matrix instructions, and 12 registers less in kernels that are held to 128.
+template <typename Act, int MT, bool PLAIN = false, bool MERGED = false> struct Sums {
     typedef typename Acc<Act>::type A;
     typedef Act act_type;
     static constexpr int ROWS = MT;
@@ -73,9 +75,10 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                                                                        // four rows (MT = 4) or one entry x eight rows (MT = 8) per
                                                                        // operand, selector of 0 / +-1.0
     static constexpr int NW = MX ? MT / 4 : 1;              // dwords per gathered slot (int8)
-    static constexpr int ND = (MX || MXF) ? MT / 4 : 1;     // result tiles
+    static_assert(!MERGED || (MT == 8 && !PLAIN), "merged result tiles belong to eight-row tiles on the matrix unit");
+    static constexpr int ND = (MX || MXF) && !MERGED ? MT / 4 : 1;  // result tiles
     v4i D[ND], Bp[ND], Bn[ND];                              // MX: 16x16 int32 result tiles and the +1 / -1 selectors
-    bool merged = false;                                    // MT = 8, columns of 32 or 64 lanes: one result tile sums lanes i, i+16 (, i+32, i+48)
+    static constexpr bool merged = MERGED;                  // one result tile sums lanes i, i+16 (, i+32, i+48)
     v4f Df[ND];                                             // MXF: the fp32 result tiles ...
     v8h Bpf[ND], Bnf[ND];                                   // ... and their selectors
     A acc[MT];
@@ -95,7 +98,6 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
 #pragma unroll
         for (int m = 0; m < MT; ++m) acc[m] = (A)0;
         if constexpr (MX) {
-            merged = MT == 8 && logL >= 5;
             // Selector held by lane j + 16 g (k-block g, output column j): 1 where the byte of the A operand
             // at the same (g, byte) position is to be added into column j.  MT = 4: A = 4 entries x 4 rows,
             // column 4 g + row.  MT = 8: A = 2 entries x 8 rows, tile x takes k-blocks 2x and 2x + 1, column
@@ -122,7 +124,6 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
         } else if constexpr (MXF) {
             // lane j + 16 g holds rows 8 g .. 8 g + 7 of selector column j.  MT = 4: the operand is two entries x four
             // rows, column 4 g + row.  MT = 8: one entry x eight rows; tiles and columns as for eight int8 rows.
-            merged = MT == 8 && logL >= 5;
             const int l = threadIdx.x & 63, g = l >> 4, j = l & 15;
 #pragma unroll
             for (int x = 0; x < ND; ++x) {
@@ -163,11 +164,7 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
                     a = v4i{(int)r[e].v[0], (int)r[e].v[1], e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[0] : 0,
                             e + 1 < NE ? (int)r[e + 1 < NE ? e + 1 : e].v[1] : 0};
                 D[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[0] : Bp[0], D[0], 0, 0, 0);
-                if constexpr (ND > 1) {
-                    // (uniform.  A loop of its own for the second tile, one branch per call instead of one per instruction,
-                    // keeps the operands alive across both loops and was slower: K=6912 N=2560, gap stream, M=8 2.0 -> 2.4 us)
-                    if (!merged) D[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[1] : Bp[1], D[1], 0, 0, 0);
-                }
+                if constexpr (ND > 1) D[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, NEG ? Bn[1] : Bp[1], D[1], 0, 0, 0);
             }
         } else if constexpr (MXF && MT == 8) {
 #pragma unroll
@@ -176,15 +173,7 @@ template <typename Act, int MT, bool PLAIN = false> struct Sums {
 #pragma unroll
                 for (int m = 0; m < 8; ++m) a[m] = r[e].v[m];
                 Df[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[0] : Bpf[0], Df[0], 0, 0, 0);
-            }
-            if (!merged) {  // (uniform; a loop of its own: one branch per call)
-#pragma unroll
-                for (int e = 0; e < NE; ++e) {
-                    v8h a;
-#pragma unroll
-                    for (int m = 0; m < 8; ++m) a[m] = r[e].v[m];
-                    Df[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[1] : Bpf[1], Df[1], 0, 0, 0);
-                }
+                if constexpr (ND > 1) Df[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, NEG ? Bnf[1] : Bpf[1], Df[1], 0, 0, 0);
             }
         } else if constexpr (MXF) {
 #pragma unroll
@@ -623,8 +612,9 @@ template <int MT> struct Quantiser {
     }
 };
 
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, bool QUANT = false>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, bool QUANT = false, bool MERGED = false>
 struct ListsBody {
+    typedef Sums<Act, MT, false, MERGED> SumsT;
     typedef typename Acc<Act>::type A;
     typedef Stager<Act, MT> St;
     static constexpr int SLOT_OF = slot_bytes<Act, MT>();
@@ -643,16 +633,16 @@ struct ListsBody {
     static constexpr int RING = TIGHT ? 4 : 8;      // rounds in flight on the generic path (8-row kernels run 10-16 wavefronts per CU and are short of registers)
     static constexpr int EARLY = MT >= 4 ? 4 : 2;     // rounds requested before the activation tile is complete (multi-row tiles take longer to stage)
 
-    static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, Sums<Act, MT> &acc)
+    static __device__ __forceinline__ void eat(const unsigned char *smem, const Round &x, u32 &runp, u32 &runq, SumsT &acc)
     {
-        consume16<Sums<Act, MT>, MODE, PRE, false>(smem, x.p, runp, acc);
-        consume16<Sums<Act, MT>, MODE, PRE, true>(smem, x.q, runq, acc);
+        consume16<SumsT, MODE, PRE, false>(smem, x.p, runp, acc);
+        consume16<SumsT, MODE, PRE, true>(smem, x.q, runq, acc);
         acc.pin();  // (and the running rows)
         if constexpr (GAPS) asm volatile("" : "+v"(runp), "+v"(runq));
     }
 
     // fp16 tiles summed on the matrix unit have a VALU twin for workgroups whose tile holds an Inf or NaN
-    static constexpr bool TWIN = Sums<Act, MT>::MXF;
+    static constexpr bool TWIN = SumsT::MXF;
     typedef Sums<Act, MT, TWIN> Plain;
 
     // One task summed on the VALU with a single round in flight (the twin's path: rare, so small rather than fast).
@@ -895,9 +885,11 @@ struct ListsBody {
             // AHEAD: while a task is walked, the next one's first rows and rounds are requested into the registers that
             // come free, so a wavefront that walks several tasks never waits with nothing in flight.  Four int8 rows
             // on gap streams only (tasks of one length, straight-line path), where it pays: headline shape, 32 GEMVs per
-            // launch, 10 tasks per wavefront 2.00 -> 1.88 us per GEMV.  Measured and left out: eight int8 rows (2.09 ->
-            // 2.29 us), four fp16 rows (2.18 -> 2.56 us), byte rows (1.70 -> 1.79 us), u16 lists (3.2 -> 13.6 us at M=4).
-            constexpr bool AHEAD = RF != 0 && !VAR && !QUANT && MT == 4 && sizeof(Act) == 1 && MODE != 0;
+            // launch, 10 tasks per wavefront 2.00 -> 1.88 us per GEMV; and eight int8 rows with one result tile, which leaves
+            // the registers for it (K=13824 N=5120 split_k=64, 14 GEMVs per launch: 8.9 -> 8.45 us; with two result tiles the
+            // kernel spilled and lost, 2.09 -> 2.29 us).  Measured and left out: four fp16 rows (2.18 -> 2.56 us), byte rows
+            // (1.70 -> 1.79 us), u16 lists (3.2 -> 13.6 us at M=4).
+            constexpr bool AHEAD = RF != 0 && !VAR && !QUANT && (MT == 4 || (MT == 8 && MERGED)) && sizeof(Act) == 1 && MODE != 0;
             const int task_next = task + task_step;
             const uint8_t *tb_next = tasks_base + (size_t)(task_next < p.tasks ? task_next : 0) * task_bytes;
             if constexpr (GAPS) {
@@ -921,7 +913,7 @@ struct ListsBody {
                 walk_plain(smem, tb, lane, n_lane, runp, runq, pacc);
                 store_lane_sums(p, pacc.acc, part, back, active, task, lane, wave, m0);
             } else {
-            Sums<Act, MT> acc;
+            SumsT acc;
             acc.init(p.logL);
 
             if constexpr (RF != 0) {
@@ -1021,38 +1013,36 @@ struct ListsBody {
             }
             if (rem) {
                 if (rem & (8 / ESZ)) {
-                    consume<Sums<Act, MT>, MODE, PRE, false, 4>(smem, t8p.x, runp, acc);
-                    consume<Sums<Act, MT>, MODE, PRE, false, 4>(smem, t8p.y, runp, acc);
-                    consume<Sums<Act, MT>, MODE, PRE, true, 4>(smem, t8q.x, runq, acc);
-                    consume<Sums<Act, MT>, MODE, PRE, true, 4>(smem, t8q.y, runq, acc);
+                    consume<SumsT, MODE, PRE, false, 4>(smem, t8p.x, runp, acc);
+                    consume<SumsT, MODE, PRE, false, 4>(smem, t8p.y, runp, acc);
+                    consume<SumsT, MODE, PRE, true, 4>(smem, t8q.x, runq, acc);
+                    consume<SumsT, MODE, PRE, true, 4>(smem, t8q.y, runq, acc);
                 }
                 if (rem & (4 / ESZ)) {
-                    consume<Sums<Act, MT>, MODE, PRE, false, 4>(smem, t4p, runp, acc);
-                    consume<Sums<Act, MT>, MODE, PRE, true, 4>(smem, t4q, runq, acc);
+                    consume<SumsT, MODE, PRE, false, 4>(smem, t4p, runp, acc);
+                    consume<SumsT, MODE, PRE, true, 4>(smem, t4q, runq, acc);
                 }
                 if (rem & (2 / ESZ)) {
-                    consume<Sums<Act, MT>, MODE, PRE, false, 2>(smem, t2p, runp, acc);
-                    consume<Sums<Act, MT>, MODE, PRE, true, 2>(smem, t2q, runq, acc);
+                    consume<SumsT, MODE, PRE, false, 2>(smem, t2p, runp, acc);
+                    consume<SumsT, MODE, PRE, true, 2>(smem, t2q, runq, acc);
                 }
                 if constexpr (ESZ == 1) {
                     if (rem & 1) {
-                        consume<Sums<Act, MT>, MODE, PRE, false, 1>(smem, t1p, runp, acc);
-                        consume<Sums<Act, MT>, MODE, PRE, true, 1>(smem, t1q, runq, acc);
+                        consume<SumsT, MODE, PRE, false, 1>(smem, t1p, runp, acc);
+                        consume<SumsT, MODE, PRE, true, 1>(smem, t1q, runq, acc);
                     }
                 }
             }
 
-            if constexpr (Sums<Act, MT>::MX || Sums<Act, MT>::MXF) {
+            if constexpr (SumsT::MX || SumsT::MXF) {
                 // Result tile x, lane l, register r: the sum of source lane 16 g + 4 (l >> 4) + r and row m, where
                 // MT = 4: g = (l >> 2) & 3, m = l & 3;  MT = 8: g = 2 x + ((l >> 3) & 1), m = l & 7.
                 // The four registers are neighbouring lanes of one column; the rest of a column's L lanes is
                 // spread over lane bits 4, 5 (the quarter) and, from L = 32, the bits that hold g.
-                constexpr int ND = Sums<Act, MT>::ND;
+                constexpr int ND = SumsT::ND;
                 const int logL = p.logL;
-                A t[ND];
-                bool merged_done = false;
-                if constexpr (MT == 8) {
-                    if (acc.merged) {
+                if constexpr (MERGED) {
+                    {
                         // one tile: lane l, register r = rows i = 4 (l >> 4) + r, result column j = l & 15 holds activation
                         // row j & 7 of the task's column j >> 3; the 16 i are the column's lanes i, i+16 (, i+32, i+48)
                         A v = acc.tile_sum(0);
@@ -1070,10 +1060,9 @@ struct ListsBody {
                         } else if (lane < MT) {
                             part[wave * MT + lane] = v;
                         }
-                        merged_done = true;
                     }
-                }
-                if (!merged_done) {
+                } else {
+                A t[ND];
 #pragma unroll
                 for (int x = 0; x < ND; ++x) {
                     t[x] = acc.tile_sum(x);
@@ -1149,11 +1138,11 @@ struct ListsBody {
 // wavefronts then walk tasks blockIdx.x*waves + wave, + gridDim.x*waves, ...
 // blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
 // exactly RF full rounds (straight-line body); RF == 0: any length (ring).
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool QUANT = false>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool QUANT = false, bool MERGED = false>
 __global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, QUANT>())) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    ListsBody<Act, MT, MODE, PRE, VAR, QUANT>::template run<RF>(p, smem);
+    ListsBody<Act, MT, MODE, PRE, VAR, QUANT, MERGED>::template run<RF>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -1165,14 +1154,14 @@ struct BatchPtrs {
     void *C[BATCH_MAX];
 };
 
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool MERGED = false>
 __global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, false>())) lists_kernel_batched(ListParams p, BatchPtrs b)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     p.w = b.w[blockIdx.z];
     p.X = b.X[blockIdx.z];
     p.C = b.C[blockIdx.z];
-    ListsBody<Act, MT, MODE, PRE, VAR>::template run<RF>(p, smem);
+    ListsBody<Act, MT, MODE, PRE, VAR, false, MERGED>::template run<RF>(p, smem);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -1191,7 +1180,7 @@ static inline int grant_lds(const void *kern, size_t lds, std::atomic<size_t> &g
     return SPTMM_OK;
 }
 
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool MERGED = false>
 static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
 {
     // Launch shape: g workgroups resident per CU, w wavefronts each.  A wavefront asks for its
@@ -1218,7 +1207,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     int regs = vgprs.load(std::memory_order_relaxed);
     if (!regs) {
         hipFuncAttributes fa;
-        hipError_t e = hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(lists_kernel<Act, MT, MODE, PRE, VAR, RF>));
+        hipError_t e = hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(lists_kernel<Act, MT, MODE, PRE, VAR, RF, false, MERGED>));
         if (e != hipSuccess) return hip_fail(e, "hipFuncGetAttributes");
         regs = fa.numRegs > 0 ? fa.numRegs : 128;
         vgprs.store(regs, std::memory_order_relaxed);
@@ -1333,7 +1322,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     dim3 grid(grid_x, (a.M + MT - 1) / MT), block(64 * wpb);
     if (a.batch) {
         {
-            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, VAR, RF>;
+            auto kern = lists_kernel_batched<Act, MT, MODE, PRE, VAR, RF, MERGED>;
             static std::atomic<size_t> lds_granted_b{48 * 1024};
             if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_b)) return rc;
             for (int first = 0; first < a.batch; first += BATCH_MAX) {
@@ -1354,7 +1343,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     }
     if (a.quant) {
         if constexpr (sizeof(Act) == 1) {
-            auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, true>;
+            auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, true, MERGED>;
             // + room for the per-wavefront sums of a full workgroup, the row maxima and the rows' 1/s
             lds = tile + (size_t)(2 * LISTS_MAX_WAVES + 1) * MT * 4;
             if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
@@ -1367,7 +1356,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             return fail(SPTMM_ERR_INVALID, "quantising launches go through the int8 kernels");
         }
     }
-    auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF>;
+    auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, false, MERGED>;
     static std::atomic<size_t> lds_granted{48 * 1024};
     if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
     hipLaunchKernelGGL(kern, grid, block, lds, st, p);
@@ -1378,6 +1367,16 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
 // Straight-line bodies exist for tasks
 // with 1, 2, 3, 4, 6 or 8 full rounds (ragged streams: for the shortest
 // task, when the longest has at most XMAX more); everything else takes the ring.
+// Eight-row tiles whose columns take 32 or 64 lanes run the kernels with one result tile (MERGED).
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF>
+static int launch_lists_g(const GemvArgs &a, hipStream_t st)
+{
+    if constexpr (MT == 8) {
+        if (a.L >= 32) return launch_lists_rf<Act, MT, MODE, PRE, VAR, RF, true>(a, st);
+    }
+    return launch_lists_rf<Act, MT, MODE, PRE, VAR, RF, false>(a, st);
+}
+
 template <typename Act, int MT, int MODE, bool PRE, bool VAR>
 static int launch_lists_t(const GemvArgs &a, hipStream_t st)
 {
@@ -1396,24 +1395,24 @@ static int launch_lists_t(const GemvArgs &a, hipStream_t st)
         if (UP_TO_THREE && rf > 3) rf = 9;  // no straight-line body of that length: falls through to the ring
         switch (rf) {
         case 0:
-            if ((VAR ? a.n_max : a.n_lane) / E16 <= ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) return launch_lists_rf<Act, MT, MODE, PRE, VAR, -1>(a, st);
+            if ((VAR ? a.n_max : a.n_lane) / E16 <= ListsBody<Act, MT, MODE, PRE, VAR>::XMAX) return launch_lists_g<Act, MT, MODE, PRE, VAR, -1>(a, st);
             break;
-        case 1: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 1>(a, st);
-        case 2: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 2>(a, st);
-        case 3: return launch_lists_rf<Act, MT, MODE, PRE, VAR, 3>(a, st);
+        case 1: return launch_lists_g<Act, MT, MODE, PRE, VAR, 1>(a, st);
+        case 2: return launch_lists_g<Act, MT, MODE, PRE, VAR, 2>(a, st);
+        case 3: return launch_lists_g<Act, MT, MODE, PRE, VAR, 3>(a, st);
         case 4:
-            if constexpr (!UP_TO_THREE) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 4>(a, st);
+            if constexpr (!UP_TO_THREE) return launch_lists_g<Act, MT, MODE, PRE, VAR, 4>(a, st);
             break;
         case 6:
-            if constexpr (!lists_short_of_registers<Act, MT>() && !UP_TO_THREE) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 6>(a, st);
+            if constexpr (!lists_short_of_registers<Act, MT>() && !UP_TO_THREE) return launch_lists_g<Act, MT, MODE, PRE, VAR, 6>(a, st);
             break;
         case 8:
-            if constexpr (!lists_short_of_registers<Act, MT>() && !UP_TO_THREE) return launch_lists_rf<Act, MT, MODE, PRE, VAR, 8>(a, st);
+            if constexpr (!lists_short_of_registers<Act, MT>() && !UP_TO_THREE) return launch_lists_g<Act, MT, MODE, PRE, VAR, 8>(a, st);
             break;
         default: break;
         }
     }
-    return launch_lists_rf<Act, MT, MODE, PRE, VAR, 0>(a, st);
+    return launch_lists_g<Act, MT, MODE, PRE, VAR, 0>(a, st);
 }
 
 template <typename Act, int MODE, bool PRE, bool VAR>
