@@ -730,6 +730,31 @@ def test_gap_stream_four_rows_batched_with_many_tasks_per_wavefront(K, N, S, spl
         o.free()
 
 
+@pytest.mark.parametrize("K,N,S,split,count,M", [
+    (6912, 2560, 4096, 32, 32, 8),    # one result tile (columns of 32 lanes), ten tasks per wavefront, rounds requested a task ahead
+    (13824, 5120, 8320, 64, 14, 8),   # columns of 64 lanes, nine tasks per wavefront, a one-entry tail
+    (6912, 2560, 4160, 32, 9, 6),
+    (2560, 640, 1536, 32, 5, 7),      # fewer tasks than wavefronts in the last workgroups
+    (2560, 6912, 1536, 16, 32, 8),    # columns of 16 lanes: two result tiles, no requests ahead
+    (6912, 2560, 4096, 8, 6, 5),      # columns of 8 lanes
+])
+def test_gap_stream_eight_rows_batched_with_many_tasks_per_wavefront(K, N, S, split, count, M):
+    test_gap_stream_four_rows_batched_with_many_tasks_per_wavefront(K, N, S, split, count, M)
+
+
+def test_gap_stream_eight_rows_single_launch_with_several_tasks_per_wavefront():
+    sp.device_init(0)
+    K, N, S = 2560, 13824, 1536
+    _, pos, neg = matrix(K, N, S)
+    for split in (16, 32, 64):
+        w = sp.Weights.upload_delta(pos, neg, K, split)
+        for M in (8, 5):
+            say("gap stream, eight rows, many tasks", split, M)
+            X = x_i8(177 + M, M, K)
+            assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), (split, M)
+        w.free()
+
+
 def test_gap_stream_four_rows_single_launch_with_several_tasks_per_wavefront():
     """A lone launch walks more than one task per wavefront when the tasks outnumber the wavefronts the chip holds."""
     sp.device_init(0)
