@@ -13,7 +13,9 @@ stream, fp16 rows); config 3 (the decoder layer's four shapes at M=1 and M=4, pe
 (K=13824 N=5120 at M=1, 8, 16, lists against i2s).  Every timed object is first checked bit-exact against the
 other encodings of the same matrix, and the CPU leg checks one GPU result per configuration against the oracle.
 
-Prints ONE JSON line (see the keys at the bottom).
+Prints ONE JSON line on stdout: the headline with its roofline and CPU baseline and one figure per configuration
+(final_line(), a few KB).  The per-row tables of every leg go to a side file (--detail, default
+gpurun_out/bench_detail.json) and, one JSON object per leg, to stderr.
 """
 import argparse
 import json
@@ -107,7 +109,88 @@ def cpu_baseline(sp_lists, gpu_headline, checks, dense_w=None, budget_s=12.0):
     }
 
 
-def main():
+# config 3 as a sequence.  (name, K, N, S, stage): the steps of a stage read the same input and do not depend on each other.
+LAYER_SEVEN = [("q", 2560, 2560, 1536, 0), ("k", 2560, 640, 1536, 0), ("v", 2560, 640, 1536, 0), ("o", 2560, 2560, 1536, 1),
+               ("gate", 2560, 6912, 1536, 2), ("up", 2560, 6912, 1536, 2), ("down", 6912, 2560, 4160, 3)]
+# the fused shapes the reference instantiates (main.cu:1107-1120: N=13824; main.cu:1916-1917: N=3840)
+LAYER_FOUR = [("qkv", 2560, 3840, 1536, 0), ("o", 2560, 2560, 1536, 1), ("gate_up", 2560, 13824, 1536, 2), ("down", 6912, 2560, 4160, 3)]
+
+
+def layer_sequence(sp, st, checks, reps):
+    """The decoder layer of config 3 timed as what it is, a sequence of launches on one stream (the loop of main.cu:767-782
+    around a whole layer instead of one kernel): 7 launches; 5 (k, v and gate, up as batched pairs); 4 with the fused shapes;
+    each also as a HIP graph, the 7 with independent projections on parallel branches.  One pass walks `layers` layers with
+    their own device copies of every matrix (more bytes than the last-level cache holds), microseconds per layer.  Outputs
+    of the first and last layer of every variant are compared across encodings, one per shape against the oracle."""
+    import numpy as np
+
+    rows, gens, seen = [], {}, {}
+    for m in (1, 4):
+        xs = {stage: sp.make_x_i8(0xC0FFEE ^ (m + 16 * stage), m, k) for stage, k in enumerate((2560, 2560, 2560, 6912))}
+        xbuf = {stage: sp.DeviceBuffer.from_numpy(x) for stage, x in xs.items()}
+        for enc in ("u16", "delta", "i2s"):
+            for label, shapes in (("seven", LAYER_SEVEN), ("four_fused", LAYER_FOUR)):
+                base, nbytes = {}, 0
+                for name, k_rows, n_cols, s_nz, stage in shapes:
+                    key = (k_rows, n_cols, s_nz)
+                    if key not in gens:
+                        gens[key] = sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)
+                    Wm, p, n = gens[key]
+                    if key not in base:
+                        base[key] = (sp.Weights.upload_u16(p, n, k_rows, 0) if enc == "u16" else
+                                     sp.Weights.upload_delta(p, n, k_rows, 0, rows=m) if enc == "delta" else sp.Weights.upload_i2s(Wm))
+                    nbytes += algorithmic_bytes(base[key].info["stream_bytes"], m, k_rows, n_cols)
+                layers = max(4, min(32, int(math.ceil(512e6 / nbytes))))
+                owned, steps, outs = list(base.values()), [], []
+                for l in range(layers):
+                    for name, k_rows, n_cols, s_nz, stage in shapes:
+                        w = base[(k_rows, n_cols, s_nz)].clone()
+                        c = sp.DeviceBuffer(4 * m * n_cols)
+                        owned += [w, c]
+                        steps.append((w, xbuf[stage], c, m, 0, 4 * l + stage))
+                        outs.append((l, name, (k_rows, n_cols, s_nz), stage, c))
+                r = {"M": m, "enc": enc, "layer": label, "launches_per_layer": len(shapes), "layers_per_pass": layers, "bytes_per_layer": nbytes,
+                     "floor_us_at_8TBps": round(nbytes / PEAK_GBPS / 1e3, 2)}
+                for mode_name, mode in sp.SEQ_MODES.items():
+                    if label == "four_fused" and mode_name in ("graph_branches", "streams", "batched_pairs"):
+                        continue  # a chain: nothing to put side by side
+                    for c in (o[-1] for o in outs):
+                        c.fill(0xFF)
+                    sp.measure_sequence(steps, max(2, reps // 10), mode, st)
+                    us = min(sp.measure_sequence(steps, reps, mode, st) for _ in range(2)) / layers
+                    r[mode_name + "_us"] = round(us, 2)
+                    # every projection of the first and the last layer: the same numbers in every encoding and variant
+                    for l, name, key, stage, c in outs:
+                        if l not in (0, layers - 1):
+                            continue
+                        got = c.to_numpy(np.int32, (m, key[1]))
+                        ref = seen.setdefault((m, key, stage), got)
+                        if ref is got:
+                            checks.append(("layer %s M=%d" % (name, m), xs[stage], gens[key][1], gens[key][2], got, key[2]))
+                        assert (got == ref).all(), ("layer sequence", enc, label, mode_name, name, l)
+                best = min(v for k, v in r.items() if k.endswith("_us") and k != "floor_us_at_8TBps")
+                r["best_us"] = best
+                r["best_pct_roofline"] = pct(nbytes, best)
+                rows.append(r)
+                for o in owned:
+                    o.free()
+        for b in xbuf.values():
+            b.free()
+    summary = {"columns": ["seven_launches_us", "five_launches_batched_pairs_us", "seven_graph_branches_us", "four_fused_launches_us", "four_fused_graph_us",
+                           "floor_us_of_seven_at_8TBps"]}
+    for m in (1, 4):
+        for enc in ("u16", "delta", "i2s"):
+            a7 = _row(rows, M=m, enc=enc, layer="seven")
+            a4 = _row(rows, M=m, enc=enc, layer="four_fused")
+            summary["M%d_%s" % (m, enc)] = [a7["launches_us"], a7["batched_pairs_us"], a7["graph_branches_us"], a4["launches_us"], a4["graph_chain_us"],
+                                            a7["floor_us_at_8TBps"]]
+    return {"rows": rows, "summary": summary,
+            "protocol": "one pass = `layers_per_pass` layers, each with its own device copy of every matrix (> 512 MB per pass: HBM-cold); "
+                        "us per layer between two HIP events around `reps` passes (sptmm_measure_sequence)"}
+
+
+def run(argv=None):
+    """-> the full result: the contract keys plus every leg's table."""
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256, help="timed steps; one step = one launch of BATCH GEMVs")
@@ -116,14 +199,18 @@ def main():
     ap.add_argument("--reps", type=int, default=0,
                     help="launches per timed loop of the legs (0: 1500, the headline shape's other encodings 4096); counter "
                          "runs under a profiler, where every launch is serialised, use a few dozen")
-    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,cfg4,density",
+    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,layer,cfg4,density",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, sync-each-call, four streams), "
                          "others (delta and i2s encodings at the headline shape), cfg1 (the same matrix at M=4), cfg2 (gap "
                          "stream with fp16 rows), cfg3 (decoder-layer shapes, M=1 and 4), cfg4 (K=13824 N=5120, M=1/8/16), "
+                         "layer (config 3 as a sequence: the decoder layer's 7 projections, or 4 with q+k+v and gate+up fused, "
+                         "issued in order / as a HIP graph, rotating over enough layers to stay HBM-cold), "
                          "density (the headline shape at 3.7-25 % nonzeros against i2s), "
                          "copy (4 launches of a 1 GiB copy kernel, for counter calibration), ceiling (a pure streaming "
                          "read of as many bytes as one step moves); profiling runs use --legs none or one leg")
-    a = ap.parse_args()
+    ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
+                    help="side file for the full result (every leg's per-row table); '' writes none")
+    a = ap.parse_args(argv)
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported "
                  "(columns shard across GPUs with no collective, but nothing here runs a second GPU)" % a.gpus)
@@ -343,6 +430,10 @@ def main():
             ww.free()
         configs["cfg4_large"] = rows
 
+    layer_seq = None
+    if "layer" in legs:
+        layer_seq = layer_sequence(sp, st, checks, a.reps or 300)
+
     density = None
     if "density" in legs:
         # Where index lists overtake the 2-bit baseline: the same shape at fewer nonzeros per column.  i2s stores
@@ -395,7 +486,7 @@ def main():
             # at BASELINE's 59 % nonzeros the lists hold 4.7x (gap stream 2.4x) the bytes of i2s; they win where they are smaller
             "beats_i2s_batched_up_to_density_pct": density["lists_beat_i2s_up_to_density_pct"] if density else None,
         },
-        "single_launch": single, "other_encodings": others, "configs": configs, "density_sweep": density,
+        "single_launch": single, "other_encodings": others, "configs": configs, "layer_sequence": layer_seq, "density_sweep": density,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_src,
@@ -409,7 +500,85 @@ def main():
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline((pos, neg), ref, checks, Wd)
     w.free()
-    print(json.dumps(out, ensure_ascii=False))
+    out["detail_file"] = os.path.relpath(a.detail, ROOT) if a.detail else None
+    return out
+
+
+def _row(rows, **want):
+    for r in rows or ():
+        if all(r.get(k) == v for k, v in want.items()):
+            return r
+    return None
+
+
+def _pick(d, *keys):
+    return {k: d[k] for k in keys if d and k in d}
+
+
+def final_line(full):
+    """The one stdout line: the contract keys, `roofline`, `cpu_baseline`, the single-launch figures, `targets`, and per
+    configuration one compact row (us per GEMV in a batched HBM-cold launch and its % of 8 TB/s, plus the lone-launch
+    HBM-cold us) -- a few KB whatever legs ran.  Everything else stays in the detail file."""
+    out = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                                 "vs_baseline", "dtype", "data", "config", "hbm_gbps", "pct_roofline", "single_launch_cold_us",
+                                 "single_launch_cold_pct_roofline", "targets", "device") if k in full}
+    rf = dict(full["roofline"])
+    src = rf.pop("traffic_source", None)
+    if src:
+        rf["traffic_measured_at_commit"] = src.get("measured_at_commit")
+        rf["traffic_file"] = os.path.relpath(TRAFFIC_SIDECAR, ROOT)
+    ceil = rf.pop("streaming_read_ceiling", None)
+    if ceil:
+        rf["streaming_read_gbps"] = ceil["gbps"]
+        rf["read_only_launch_us"] = _pick(ceil.get("per_launch_read"), "cold_us", "warm_us")
+    out["roofline"] = rf
+    if "cpu_baseline" in full:
+        out["cpu_baseline"] = full["cpu_baseline"]
+    if full.get("single_launch"):
+        out["single_launch"] = full["single_launch"]
+
+    def brief(r):  # [us per GEMV batched, % of 8 TB/s batched, us alone HBM-cold]
+        return [r["batched_us"], r["batched_pct_roofline"], r["alone_cold_us"]] if r else None
+
+    summary = {"columns": ["batched_us_per_gemv", "batched_pct_of_8TBps", "one_per_launch_cold_us"]}
+    oth = full.get("other_encodings") or {}
+    if oth:
+        summary["cfg0_other_encodings"] = {k: brief(v) for k, v in oth.items()}
+    cf = full.get("configs") or {}
+    if "cfg1_m4" in cf:
+        summary["cfg1_m4"] = {e: brief(_row(cf["cfg1_m4"], enc=e)) for e in ("u16", "delta", "i2s")}
+    if "cfg2_delta_fp16" in cf:
+        summary["cfg2_delta_fp16"] = {"M%d" % r["M"]: brief(r) for r in cf["cfg2_delta_fp16"]}
+    if "cfg3_layer" in cf:
+        summary["cfg3_layer_summed"] = {"M%d_%s" % (t["M"], t["enc"]): [t["batched_us"], t["batched_pct_roofline"], t["alone_cold_us"]]
+                                        for t in cf["cfg3_layer"]["summed_layer"]}
+    if "cfg4_large" in cf:
+        summary["cfg4_large"] = {"M%d_%s" % (r["M"], r["enc"].replace(" ", "_")): brief(r) for r in cf["cfg4_large"]}
+    if full.get("layer_sequence"):
+        summary["layer_sequence"] = full["layer_sequence"]["summary"]
+    dn = full.get("density_sweep")
+    if dn:
+        summary["density_lists_over_i2s"] = {str(c["density_pct"]): c["lists_over_i2s"] for c in dn["against_i2s"]}
+    out["summary"] = summary
+    out["detail_file"] = full.get("detail_file")
+    return json.dumps(out, ensure_ascii=False, separators=(",", ":"))
+
+
+def main():
+    full = run()
+    path = full.get("detail_file")
+    if path:
+        path = os.path.join(ROOT, path)
+        try:
+            os.makedirs(os.path.dirname(path), exist_ok=True)
+            with open(path, "w") as f:
+                json.dump(full, f, ensure_ascii=False, indent=1)
+        except OSError as e:  # a read-only tree: the tables still go to stderr
+            print("bench.py: cannot write %s: %s" % (path, e), file=sys.stderr)
+    for leg in ("single_launch", "other_encodings", "configs", "layer_sequence", "density_sweep"):
+        if full.get(leg):
+            print(json.dumps({leg: full[leg]}, ensure_ascii=False), file=sys.stderr)
+    print(final_line(full), flush=True)
 
 
 if __name__ == "__main__":

@@ -280,6 +280,12 @@ int sptmm_event_destroy(void *event);
 int sptmm_event_record(void *event, void *stream);
 int sptmm_event_sync(void *event);
 int sptmm_event_elapsed_us(void *start, void *stop, double *us);
+/* Work issued on `stream` after this call waits for what `event` had recorded.  Between
+ * sptmm_graph_begin and _end it is also how a second stream joins the capture and leaves it
+ * again: record an event on the capturing stream and let the side stream wait for it (fork),
+ * launch on both, record an event on the side stream and let the capturing stream wait for it
+ * (join) -- independent projections then sit on parallel branches of the graph. */
+int sptmm_stream_wait_event(void *stream, void *event);
 /* Stream capture: the launches issued on `stream` between _begin and _end (any of
  * the sptmm_gemv_* calls, in any mix) become one executable HIP graph that
  * _launch replays -- a decoder layer's fixed sequence of projections as one
@@ -308,6 +314,29 @@ int sptmm_graph_destroy(void *graph);
  * events recorded on that stream. */
 int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X_dev, int M, void *C_dev,
                        int iters, int mode, void *stream, double *us_per_call);
+/* The same loop around a SEQUENCE of GEMVs -- a decoder layer's projections in their order
+ * (the per-shape loops of main.cu:994-1459 time each projection on its own).  steps[i] is one
+ * GEMV (act: 0 int8, 1 fp16, 2 fp32); `stage` is non-decreasing over the array, stages run in
+ * order, and the steps of one stage do not depend on each other (q, k, v of one input).  One
+ * pass over all n_steps is one sequence; it is issued `reps` times between two events on
+ * `stream` (made by sptmm_stream_create), after one untimed pass.  mode:
+ *   0  every step its own launch, in array order, on `stream`
+ *   1  one pass captured into a HIP graph as a chain, replayed `reps` times
+ *   2  captured with the steps of a stage on parallel branches of the graph (fork / join)
+ *   3  no graph; the steps of a stage issued on side streams that fork from and join `stream`
+ *   4  as 0, but neighbouring steps of one stage whose streams agree in kind and shape (and in M
+ *      and act) go out as ONE batched launch (sptmm_gemv_batched)
+ * Reports mean microseconds per sequence.  Weights of several layers in one array (stages
+ * numbered through) keep the pass larger than the last-level cache. */
+typedef struct sptmm_step {
+    const sptmm_weights *w;
+    const void *X_dev;
+    void *C_dev;
+    int M;
+    int act;
+    int stage;
+} sptmm_step;
+int sptmm_measure_sequence(const sptmm_step *steps, int n_steps, int reps, int mode, void *stream, double *us_per_sequence);
 /* Reads `bytes` of a scratch buffer and writes them back (a plain copy kernel):
  * evicts cached weight streams between cold-read timings and calibrates the
  * traffic counters. */

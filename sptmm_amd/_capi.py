@@ -11,10 +11,12 @@ __all__ = [
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
     "generate_ternary_iid", "dense_from_i2s_words", "choose_split_k", "wide_k_tile", "pack_wide", "unpack_wide",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
-    "device_sync", "Graph", "measure_gemv", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
+    "device_sync", "Graph", "measure_gemv", "measure_sequence", "Step", "SEQ_MODES", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
 
 KIND_U16, KIND_DELTA, KIND_I2S = 1, 2, 3
+# modes of sptmm_measure_sequence
+SEQ_MODES = {"launches": 0, "graph_chain": 1, "graph_branches": 2, "streams": 3, "batched_pairs": 4}
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
@@ -36,6 +38,7 @@ EXPORTS = [
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
     "sptmm_graph_begin", "sptmm_graph_end", "sptmm_graph_launch", "sptmm_graph_destroy",
+    "sptmm_stream_wait_event", "sptmm_measure_sequence",
 ]
 
 
@@ -55,6 +58,11 @@ class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
                 ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64),
                 ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int), ("row_bytes", C.c_int), ("stones", C.c_int)]
+
+
+class Step(C.Structure):
+    """sptmm_step: one GEMV of a sequence (see sptmm_measure_sequence)."""
+    _fields_ = [("w", C.c_void_p), ("X_dev", C.c_void_p), ("C_dev", C.c_void_p), ("M", C.c_int), ("act", C.c_int), ("stage", C.c_int)]
 
 
 def lib_path() -> str:
@@ -111,6 +119,8 @@ def lib() -> C.CDLL:
         L.sptmm_graph_launch.argtypes = [C.c_void_p, C.c_void_p]
         L.sptmm_graph_destroy.argtypes = [C.c_void_p]
         L.sptmm_event_elapsed_us.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]
+        L.sptmm_stream_wait_event.argtypes = [C.c_void_p, C.c_void_p]
+        L.sptmm_measure_sequence.argtypes = [C.POINTER(Step), C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         _LIB = L
     return _LIB
 
@@ -338,6 +348,10 @@ class Stream:
     def sync(self):
         _ck(lib().sptmm_stream_sync(self.handle))
 
+    def wait(self, event: "Event"):
+        """Later work on this stream waits for what `event` recorded (inside a capture: joins / leaves the capture)."""
+        _ck(lib().sptmm_stream_wait_event(self.handle, event.handle))
+
     def destroy(self):
         if self.handle:
             lib().sptmm_stream_destroy(self.handle)
@@ -412,6 +426,14 @@ def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuff
     finally:
         if own:
             stream.destroy()
+    return us.value
+
+
+def measure_sequence(steps, reps: int, mode: int, stream: "Stream") -> float:
+    """Mean microseconds per pass over `steps` = [(weights, X buffer, C buffer, M, act, stage), ...] (see sptmm_measure_sequence)."""
+    arr = (Step * len(steps))(*[Step(w.handle, x.ptr, c.ptr, m, act, stage) for w, x, c, m, act, stage in steps])
+    us = C.c_double()
+    _ck(lib().sptmm_measure_sequence(arr, len(steps), reps, mode, stream.handle, C.byref(us)))
     return us.value
 
 

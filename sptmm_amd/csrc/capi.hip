@@ -161,16 +161,11 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     // behind its count table exactly like a stream of balanced lists (the packers share slot_offset()): it runs on the
     // kernels for tasks of one length -- no table look-ups, straight-line bodies of the exact length (K=6912 N=2560, 864
     // entries per list, 32 GEMVs per launch: 0.81 -> 0.75 us per GEMV).
-    std::vector<const void *> behind_table;
     if (a.ragged && a.n_min == a.n_max && !a.stones && w->info.kind != SPTMM_KIND_I2S) {
         a.ragged = 0;
         a.n_lane = a.n_max;
         a.w = (const uint8_t *)w->dev + w->counts_bytes;
-        if (batch) {
-            behind_table.resize(batch);
-            for (int i = 0; i < batch; ++i) behind_table[i] = (const uint8_t *)bw[i] + w->counts_bytes;
-            a.batch_w = behind_table.data();
-        }
+        a.batch_w_skip = (size_t)w->counts_bytes;  // (the list launchers add it to every stream of a batch)
     }
     switch (w->info.kind) {
     case SPTMM_KIND_U16: return launch_u16(a, act, stream);
@@ -724,6 +719,12 @@ int sptmm_event_elapsed_us(void *a, void *b, double *us)
     *us = (double)ms * 1000.0;
     return SPTMM_OK;
 }
+int sptmm_stream_wait_event(void *s, void *ev)
+{
+    if (!ev) return fail(SPTMM_ERR_INVALID, "null pointer");
+    HIP_TRY(hipStreamWaitEvent((hipStream_t)s, (hipEvent_t)ev, 0));
+    return SPTMM_OK;
+}
 struct sptmm_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -893,7 +894,156 @@ done:
 }
 }  // namespace
 
+namespace {
+bool same_batch_shape(const sptmm_weights *a, const sptmm_weights *b)
+{
+    const sptmm_winfo &x = a->info, &y = b->info;
+    return x.kind == y.kind && x.K == y.K && x.N == y.N && x.S == y.S && x.split_k == y.split_k && x.delta_bits == y.delta_bits &&
+           x.ragged == y.ragged && x.k_tile == y.k_tile && x.row_bytes == y.row_bytes && x.stones == y.stones && a->wide == b->wide &&
+           (!a->wide || memcmp(&a->wh, &b->wh, sizeof(WideHeader)) == 0) && a->task_stride == b->task_stride && a->n_min == b->n_min;
+}
+
+int measure_sequence(const sptmm_step *steps, int n, int reps, int mode, void *stream, double *us)
+{
+    if (!steps || n < 1 || reps < 1 || !us) return fail(SPTMM_ERR_INVALID, "bad argument");
+    if (mode < 0 || mode > 4) return fail(SPTMM_ERR_INVALID, "mode must be 0..4");
+    if (!stream) return fail(SPTMM_ERR_INVALID, "sptmm_measure_sequence needs a stream made by sptmm_stream_create");
+    int widest = 1;
+    for (int i = 0, run = 0; i < n; ++i) {
+        if (!steps[i].w || !steps[i].X_dev || !steps[i].C_dev || steps[i].M < 1 || steps[i].act < ACT_I8 || steps[i].act > ACT_F32)
+            return fail(SPTMM_ERR_INVALID, "bad step %d", i);
+        if (i > 0 && steps[i].stage < steps[i - 1].stage) return fail(SPTMM_ERR_INVALID, "stages must not decrease (step %d)", i);
+        run = i > 0 && steps[i].stage == steps[i - 1].stage ? run + 1 : 1;
+        widest = std::max(widest, run);
+    }
+    constexpr int MAX_SIDE = 7;
+    if (widest > MAX_SIDE + 1) return fail(SPTMM_ERR_UNSUPPORTED, "at most %d steps per stage", MAX_SIDE + 1);
+    const bool fork = mode == 2 || mode == 3, graphed = mode == 1 || mode == 2;
+    hipStream_t st = (hipStream_t)stream;
+    hipStream_t side[MAX_SIDE] = {};
+    hipEvent_t forked = nullptr, joined[MAX_SIDE] = {}, e0 = nullptr, e1 = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int rc = SPTMM_OK;
+    float ms = 0.f;
+    auto bail = [&](hipError_t e, const char *what) { rc = hip_fail(e, what); };
+#define M_TRY(expr)                        \
+    do {                                   \
+        hipError_t e_ = (expr);            \
+        if (e_ != hipSuccess) {            \
+            bail(e_, #expr);               \
+            goto done;                     \
+        }                                  \
+    } while (0)
+    // one pass over the steps: stage by stage, in array order
+    auto pass = [&]() -> int {
+        for (int i = 0; i < n;) {
+            int j = i + 1;
+            while (j < n && steps[j].stage == steps[i].stage) ++j;
+            if (fork && j - i > 1) {
+                hipError_t e = hipEventRecord(forked, st);
+                for (int b = 1; b < j - i && e == hipSuccess; ++b) e = hipStreamWaitEvent(side[b - 1], forked, 0);
+                if (e != hipSuccess) return hip_fail(e, "forking the stage");
+                for (int b = 0; b < j - i; ++b) {
+                    const sptmm_step &s = steps[i + b];
+                    if (int r = gemv_common(s.w, s.X_dev, s.M, s.C_dev, b ? side[b - 1] : st, (ActType)s.act)) return r;
+                }
+                for (int b = 1; b < j - i && e == hipSuccess; ++b) {
+                    e = hipEventRecord(joined[b - 1], side[b - 1]);
+                    if (e == hipSuccess) e = hipStreamWaitEvent(st, joined[b - 1], 0);
+                }
+                if (e != hipSuccess) return hip_fail(e, "joining the stage");
+            } else {
+                for (int b = i; b < j;) {
+                    int c = b + 1;
+                    if (mode == 4)
+                        while (c < j && c - b < 32 && steps[c].M == steps[b].M && steps[c].act == steps[b].act && same_batch_shape(steps[b].w, steps[c].w)) ++c;
+                    if (c - b > 1) {
+                        const sptmm_weights *ws[32];
+                        const void *xs[32];
+                        void *cs[32];
+                        for (int k = b; k < c; ++k) ws[k - b] = steps[k].w, xs[k - b] = steps[k].X_dev, cs[k - b] = steps[k].C_dev;
+                        if (int r = sptmm_gemv_batched(ws, xs, cs, c - b, steps[b].M, steps[b].act, st)) return r;
+                    } else {
+                        const sptmm_step &s = steps[b];
+                        if (int r = gemv_common(s.w, s.X_dev, s.M, s.C_dev, st, (ActType)s.act)) return r;
+                    }
+                    b = c;
+                }
+            }
+            i = j;
+        }
+        return SPTMM_OK;
+    };
+    M_TRY(hipEventCreate(&e0));
+    M_TRY(hipEventCreate(&e1));
+    if (fork) {
+        M_TRY(hipEventCreateWithFlags(&forked, hipEventDisableTiming));
+        for (int b = 0; b < widest - 1; ++b) {
+            M_TRY(hipStreamCreateWithFlags(&side[b], hipStreamNonBlocking));
+            M_TRY(hipEventCreateWithFlags(&joined[b], hipEventDisableTiming));
+        }
+    }
+    if (graphed) {
+        M_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        rc = pass();
+        hipError_t ce = hipStreamEndCapture(st, &graph);
+        if (rc != SPTMM_OK) goto done;
+        M_TRY(ce);
+        M_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        M_TRY(hipGraphLaunch(exec, st));
+        M_TRY(hipStreamSynchronize(st));
+        M_TRY(hipEventRecord(e0, st));
+        for (int r = 0; r < reps; ++r) M_TRY(hipGraphLaunch(exec, st));
+    } else {
+        rc = pass();
+        if (rc != SPTMM_OK) goto done;
+        M_TRY(hipStreamSynchronize(st));
+        M_TRY(hipEventRecord(e0, st));
+        for (int r = 0; r < reps; ++r) {
+            rc = pass();
+            if (rc != SPTMM_OK) goto done;
+        }
+    }
+    M_TRY(hipEventRecord(e1, st));
+    M_TRY(hipEventSynchronize(e1));
+    M_TRY(hipEventElapsedTime(&ms, e0, e1));
+    *us = (double)ms * 1000.0 / reps;
+done:
+#undef M_TRY
+    if (rc != SPTMM_OK) {
+        // a capture that failed half way is ended so that the stream is usable again
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+            hipGraph_t dead = nullptr;
+            (void)hipStreamEndCapture(st, &dead);
+            if (dead) (void)hipGraphDestroy(dead);
+        }
+        (void)hipGetLastError();
+    }
+    (void)hipStreamSynchronize(st);
+    for (int b = 0; b < MAX_SIDE; ++b) {
+        if (side[b]) {
+            (void)hipStreamSynchronize(side[b]);
+            (void)hipStreamDestroy(side[b]);
+        }
+        if (joined[b]) (void)hipEventDestroy(joined[b]);
+    }
+    if (forked) (void)hipEventDestroy(forked);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return rc;
+}
+}  // namespace
+
 extern "C" {
+
+int sptmm_measure_sequence(const sptmm_step *steps, int n_steps, int reps, int mode, void *stream, double *us_per_sequence)
+{
+    return guarded([&]() -> int { return measure_sequence(steps, n_steps, reps, mode, stream, us_per_sequence); });
+}
 
 int sptmm_measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters,
                        int mode, void *stream, double *us_per_call)

@@ -172,6 +172,7 @@ struct GemvArgs {
     // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each
     int batch = 0;
     const void *const *batch_w = nullptr;
+    size_t batch_w_skip = 0;  // bytes in front of every batch_w[i] that the kernels do not read (a count table they need not look at)
     const void *const *batch_X = nullptr;
     void *const *batch_C = nullptr;
 };

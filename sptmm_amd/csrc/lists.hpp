@@ -1329,7 +1329,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
                 BatchPtrs b{};
                 const int n = a.batch - first < BATCH_MAX ? a.batch - first : BATCH_MAX;
                 for (int i = 0; i < n; ++i) {
-                    b.w[i] = (const uint8_t *)a.batch_w[first + i];
+                    b.w[i] = (const uint8_t *)a.batch_w[first + i] + a.batch_w_skip;
                     b.X[i] = a.batch_X[first + i];
                     b.C[i] = a.batch_C[first + i];
                 }

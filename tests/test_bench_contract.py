@@ -14,17 +14,51 @@ def test_more_than_one_gpu_is_refused():
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
 
 
+CONTRACT_KEYS = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+                 "dtype", "data", "config", "roofline")
+LINE_LIMIT = 6000  # characters of the one stdout line: what reads the line keeps a bounded tail of stdout
+
+
+def test_final_line_of_a_full_run_is_short_and_keeps_the_contract():
+    """The line bench.py prints is built by final_line() from the full result.  With every default leg in the result
+    (tests/golden/bench_full_sample.json: a full default run of this bench on an MI355X) it stays a few KB and still
+    carries the contract keys, the roofline and the CPU baseline; the per-row tables stay out of it."""
+    sys.path.insert(0, ROOT)
+    import bench
+
+    full = json.load(open(os.path.join(ROOT, "tests", "golden", "bench_full_sample.json")))
+    for leg in ("single_launch", "other_encodings", "configs", "density_sweep", "cpu_baseline", "layer_sequence"):
+        assert full.get(leg), leg
+    assert len(json.dumps(full)) > 4 * LINE_LIMIT  # the sample really holds the tables
+    line = bench.final_line(full)
+    assert len(line) < LINE_LIMIT and "\n" not in line
+    j = json.loads(line)
+    for k in CONTRACT_KEYS + ("cpu_baseline", "targets", "summary", "single_launch_cold_us"):
+        assert k in j, k
+    for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "launch_us"):
+        assert k in j["roofline"], k
+    for k in ("value", "unit", "cores", "kind", "sample"):
+        assert k in j["cpu_baseline"], k
+    assert "configs" not in j and "density_sweep" not in j
+    for k in ("cfg1_m4", "cfg2_delta_fp16", "cfg3_layer_summed", "cfg4_large", "layer_sequence", "density_lists_over_i2s"):
+        assert k in j["summary"], k
+
+
 @pytest.mark.gpu
-def test_json_line_has_the_contract_keys():
-    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "8", "--warmup", "2", "--no-cpu", "--legs", "ceiling"],
-                       capture_output=True, text=True, timeout=600)
+def test_json_line_has_the_contract_keys(tmp_path):
+    detail = str(tmp_path / "detail.json")
+    # every default leg, with short timing loops: the line that is checked is the line a default run prints
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "8", "--warmup", "2", "--no-cpu", "--reps", "48",
+                        "--detail", detail], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if l.strip()]
-    assert len(lines) == 1
+    assert len(lines) == 1 and len(lines[0]) < LINE_LIMIT
     j = json.loads(lines[0])
-    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
-              "dtype", "data", "config", "roofline"):
+    for k in CONTRACT_KEYS:
         assert k in j, k
+    full = json.load(open(detail))
+    assert full["configs"]["cfg3_layer"]["shapes"] and full["density_sweep"]["shapes"] and full["layer_sequence"]["rows"]
+    assert "layer_sequence" in j["summary"] and "cfg4_large" in j["summary"]
     assert j["n_gpus"] == 1 and j["steps"] == 8 and j["warmup"] == 2 and j["higher_is_better"] is False and j["vs_baseline"] is None
     assert "workload" in j["config"] and "model" not in j["config"]
     rf = j["roofline"]
@@ -33,7 +67,7 @@ def test_json_line_has_the_contract_keys():
     assert abs(j["value"] * 32 - rf["launch_us"]) < 0.05 * rf["launch_us"]
     assert 0.5 < rf["frac_of_streaming_read"] < 1.3
     side = json.load(open(os.path.join(ROOT, "profiles", "traffic_lists_kernel_batched_i8_u16_cfg0.json")))
-    assert rf["traffic"] == side["traffic_bytes_per_launch"] and rf["traffic_source"]["measured_at_commit"] == side["measured_at_commit"]
+    assert rf["traffic"] == side["traffic_bytes_per_launch"] and rf["traffic_measured_at_commit"] == side["measured_at_commit"]
     assert rf["algorithmic_bytes_per_launch"] == side["algorithmic_bytes_per_launch"]
 
 
