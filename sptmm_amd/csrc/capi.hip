@@ -340,8 +340,9 @@ int sptmm_weights_upload_wide(const int8_t *W, int K, int N, int kind, int split
         if (int rc = device_caps(&caps)) return rc;
         const int k_tile = sptmm_wide_k_tile(K, caps.lds);
         if (k_tile < 0) return k_tile;
+        if (split_k > 64) return fail(SPTMM_ERR_INVALID, "wide streams take split_k 8, 16, 32 or 64 (or 0: the library's pick), not %d", split_k);
         if (int rc = resolve_split_dense(W, K, N, kind, &split_k)) return rc;
-        if (split_k > 64) split_k = 64;
+        if (split_k > 64) split_k = 64;  // (the automatic choice may name a split the ordinary streams take)
         int bits = 0;
         size_t read_bytes = 0;
         uint64_t nnz = 0;

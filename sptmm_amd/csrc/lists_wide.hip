@@ -264,12 +264,17 @@ template <typename Act, int MODE, int RING_ = 4> struct WideBody {
         }
     }
 
-    // C[m][col] = (or +=, behind the first phase) v; the same lane writes the same element in every phase
+    // C[m][col] = (or +=, behind the first phase) v.  An element is written by the same WAVEFRONT in every phase (a task
+    // keeps its wavefront), by the same lane as long as the phases sum on the same unit; where an fp16 tile holds a
+    // non-finite value and the phase sums on the vector unit, another lane of that wavefront writes it.  Either way the
+    // earlier store is complete and in L2 before the later load: every phase but the first starts with a workgroup
+    // barrier, which waits for the wavefront's outstanding stores, and both the store and the load are agent-scope
+    // atomics (relaxed), which go to L2 rather than stay in the compute unit's own cache.
     static __device__ __forceinline__ void put(const WideParams &p, void *C, int m, int col, A v, bool first)
     {
         A *c = reinterpret_cast<A *>(C) + (size_t)m * p.N + col;
-        if (!first) v += __hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // from L2, where this lane's own store went
-        *c = v;
+        if (!first) v += __hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(c, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // (w, Xv, C: the launch's stream, activations and output; a batched launch picks them per blockIdx.z and leaves

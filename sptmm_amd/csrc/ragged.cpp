@@ -250,10 +250,13 @@ void pack_u16(const RaggedPlan &pl, uint8_t *stream)
 // Lane v of a column owns entries [v*n, (v+1)*n) of the sorted list; where the list ends the lane
 // steps to the zero row K and stays there (gap 0), and the lanes behind it start on K.  16-bit
 // gaps follow the sorted order; 8-bit gaps are signed and follow the bank-aware order.
-void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
+// False when the scheduler refused some task's runs (a step that does not fit a signed byte): that task's stream is
+// then unwritten and the whole stream must not be used.
+bool pack_gaps(const RaggedPlan &pl, uint8_t *stream)
 {
     const Geometry &g = pl.g;
     uint8_t *base = stream + pl.counts_bytes;
+    std::vector<uint8_t> bad(g.tasks, 0);
     parallel_for(g.tasks, [&](int task) {
         const int n = pl.n_task[task];
         uint8_t *t = base + (size_t)task * pl.stride;
@@ -272,7 +275,7 @@ void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
                     r.resize(n, (uint16_t)rest);
                 }
             }
-            write_task_runs8(t, n, 65535, rows, pl.bank_shift);
+            if (!write_task_runs8(t, n, 65535, rows, pl.bank_shift)) bad[task] = 1;
             return;
         }
         for (int sign = 0; sign < 2; ++sign)
@@ -284,7 +287,7 @@ void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
                 for (int i = 0; i < n; ++i) r[i] = first + i < cnt ? e[first + i] : (uint16_t)pl.K;
             }
         if (pl.esz == 1) {
-            write_task_runs8(t, n, pl.K, rows, pl.bank_shift);  // the plan has checked that every gap fits
+            if (!write_task_runs8(t, n, pl.K, rows, pl.bank_shift)) bad[task] = 1;  // (the plan has checked that every gap fits)
         } else {
             for (int sign = 0; sign < 2; ++sign)
                 for (int lane = 0; lane < 64; ++lane) {
@@ -295,6 +298,9 @@ void pack_gaps(const RaggedPlan &pl, uint8_t *stream)
         }
     });
     put_counts(pl, stream);
+    for (uint8_t b : bad)
+        if (b) return false;
+    return true;
 }
 
 }  // namespace
@@ -378,8 +384,8 @@ int sptmm_pack_ragged_rows(const int8_t *W, int K, int N, int kind, int split_k,
         memset(out, 0, pl.counts_bytes + pl.stride * pl.g.tasks);
         if (kind == SPTMM_KIND_U16)
             pack_u16(pl, (uint8_t *)out);
-        else
-            pack_gaps(pl, (uint8_t *)out);
+        else if (!pack_gaps(pl, (uint8_t *)out))
+            return fail(SPTMM_ERR_INVALID, "a run of the gap stream has a step that does not fit a signed byte");
         return SPTMM_OK;
     });
 }

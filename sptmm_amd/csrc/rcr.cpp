@@ -9,16 +9,25 @@
 //
 // Unlike the reference, any shape that passes its own validity rules runs (there
 // is no table of compiled-in shapes), activations are seeded, and results are
-// checked: the three encodings of the same matrix must agree.
+// checked: every method's device output is compared with a gather-sum over the
+// same lists computed here on the host ("# check=PASS"), and that host loop is
+// timed on the cores this process may use ("# cpu: ...").  -cpu_only runs the
+// host side alone (no device needed): the CPU line, and the gather-sum checked
+// against the plain dense product of the same matrix.
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
+#include <chrono>
 #include <iostream>
 #include <string>
+#include <thread>
 #include <vector>
+
+#include <sched.h>
 
 #include "../../include/sptmm.h"
 
@@ -26,6 +35,8 @@ namespace {
 
 struct Flags {
     bool cu_blas = false, i2s = false, check = true, help = false;
+    bool cpu = true;        // time the host gather-sum and print the "# cpu:" line
+    bool cpu_only = false;  // host side only: no device is touched
     uint64_t row_split3_small = 0, row_split_delta2 = 0;
     uint64_t M = 32, K = 3072, N = 768, S = 256, L = 1;  // defaults of main.cu:43-47
     uint32_t iter = 10;
@@ -69,7 +80,7 @@ void parse(int argc, char **argv, Flags &f)
         int kind;  // 0 bool, 1 u64, 2 u32, 3 string
         void *dst;
     } specs[] = {
-        {"cu_blas", 0, &f.cu_blas}, {"i2s", 0, &f.i2s}, {"check", 0, &f.check}, {"help", 0, &f.help},
+        {"cu_blas", 0, &f.cu_blas}, {"i2s", 0, &f.i2s}, {"check", 0, &f.check}, {"help", 0, &f.help}, {"cpu", 0, &f.cpu}, {"cpu_only", 0, &f.cpu_only},
         {"row_split3_small", 1, &f.row_split3_small}, {"row_split_delta2", 1, &f.row_split_delta2},
         {"M", 1, &f.M}, {"K", 1, &f.K}, {"N", 1, &f.N}, {"S", 1, &f.S}, {"L", 1, &f.L},
         {"iter", 2, &f.iter}, {"cold", 1, &f.cold}, {"seed", 1, &f.seed}, {"act", 3, &f.act},
@@ -177,6 +188,132 @@ void make_x_normal(uint32_t seed, size_t n, std::vector<float> &out)
     }
 }
 
+float half_to_float(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    uint32_t b;
+    if (e == 0) {
+        if (!m) {
+            b = sign;
+        } else {  // subnormal: value = m * 2^-24
+            float v = (float)m * 5.9604644775390625e-8f;
+            memcpy(&b, &v, 4);
+            b |= sign;
+        }
+    } else if (e == 31) {
+        b = sign | 0x7f800000u | (m << 13);
+    } else {
+        b = sign | ((e + 112u) << 23) | (m << 13);
+    }
+    float f;
+    memcpy(&f, &b, 4);
+    return f;
+}
+
+// cores this process may run on
+int affinity_cores()
+{
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    if (sched_getaffinity(0, sizeof set, &set) != 0) return 1;
+    const int n = CPU_COUNT(&set);
+    return n > 0 ? n : 1;
+}
+
+// body(c0, c1) over [0, n) split statically across `threads` threads
+template <class F> void over_columns(int n, int threads, F body)
+{
+    if (threads <= 1) {
+        body(0, n);
+        return;
+    }
+    std::vector<std::thread> th;
+    for (int t = 0; t < threads; ++t) th.emplace_back([=] { body((int)((long)n * t / threads), (int)((long)n * (t + 1) / threads)); });
+    for (auto &t : th) t.join();
+}
+
+// All threads meet here between repetitions of a timed loop (the workers live for the whole loop, so that no
+// repetition pays for starting them).
+struct SpinBarrier {
+    explicit SpinBarrier(int n) : n_(n) {}
+    void wait()
+    {
+        const int gen = gen_.load(std::memory_order_acquire);
+        if (count_.fetch_add(1, std::memory_order_acq_rel) + 1 == n_) {
+            count_.store(0, std::memory_order_relaxed);
+            gen_.fetch_add(1, std::memory_order_release);
+        } else {
+            int spins = 0;
+            while (gen_.load(std::memory_order_acquire) == gen)
+                if (++spins > 2000) std::this_thread::yield();
+        }
+    }
+    const int n_;
+    std::atomic<int> count_{0}, gen_{0};
+};
+
+// `reps` calls of body(c0, c1) over [0, n) on `threads` persistent threads; microseconds of every call (barrier to barrier)
+template <class F> std::vector<double> timed_over_columns(int n, int threads, int max_reps, double budget_s, F body)
+{
+    typedef std::chrono::steady_clock clk;
+    std::vector<double> t;
+    SpinBarrier bar(threads);
+    std::atomic<bool> stop{false};
+    auto worker = [&](int id) {
+        const int c0 = (int)((long)n * id / threads), c1 = (int)((long)n * (id + 1) / threads);
+        const auto begin = clk::now();
+        for (int rep = -3;; ++rep) {  // three warm-ups
+            bar.wait();
+            const auto t0 = clk::now();
+            if (stop.load(std::memory_order_acquire)) break;
+            body(c0, c1);
+            bar.wait();
+            if (id == 0) {
+                const auto t1 = clk::now();
+                if (rep >= 0) t.push_back(std::chrono::duration<double, std::micro>(t1 - t0).count());
+                if ((int)t.size() >= max_reps || ((int)t.size() >= 3 && std::chrono::duration<double>(t1 - begin).count() > budget_s))
+                    stop.store(true, std::memory_order_release);
+            }
+        }
+    };
+    std::vector<std::thread> th;
+    for (int i = 1; i < threads; ++i) th.emplace_back(worker, i);
+    worker(0);
+    for (auto &x : th) x.join();
+    return t;
+}
+
+// The reference kernel's sum on the host (main.cu:577-593): C[m][n] = sum X[m][pos(n)] - sum X[m][neg(n)],
+// int32 for int8 rows, double for float rows.  X is [M][K] of T; out is [M][N].
+template <class T, class A, class Conv>
+void host_gather_columns(const T *X, int M, int K, int N, int half, const uint16_t *pos, const uint16_t *neg, int c0, int c1, A *out, Conv conv)
+{
+    for (int m = 0; m < M; ++m) {
+        const T *x = X + (size_t)m * K;
+        for (int c = c0; c < c1; ++c) {
+            const uint16_t *p = pos + (size_t)c * half, *q = neg + (size_t)c * half;
+            A acc = 0;
+            for (int i = 0; i < half; ++i) acc += (A)conv(x[p[i]]) - (A)conv(x[q[i]]);
+            out[(size_t)m * N + c] = acc;
+        }
+    }
+}
+
+// the textbook product with the dense matrix (column n at W + n*K): the host's own second opinion on the lists
+template <class T, class A, class Conv>
+void host_dense_product(const T *X, int M, int K, int N, const int8_t *W, int threads, A *out, Conv conv)
+{
+    over_columns(N, threads, [=](int c0, int c1) {
+        for (int m = 0; m < M; ++m)
+            for (int c = c0; c < c1; ++c) {
+                const int8_t *w = W + (size_t)c * K;
+                A acc = 0;
+                for (int k = 0; k < K; ++k) acc += (A)conv(X[(size_t)m * K + k]) * (A)w[k];
+                out[(size_t)m * N + c] = acc;
+            }
+    });
+}
+
 struct Method {
     const char *label;
     sptmm_weights *w;
@@ -196,7 +333,8 @@ int main(int argc, char **argv)
                "  -i2s                        2-bit packed dense-ternary baseline\n"
                "  -cu_blas                    not available in this layout (aborts like the reference's rcr)\n"
                "  -M -K -N -S -L -iter        shape, nonzeros per column, iterations\n"
-               "  -act i8|f16|f32  -seed <n>  -cold <copies>  -nocheck\n");
+               "  -act i8|f16|f32  -seed <n>  -cold <copies>  -nocheck  -nocpu (no host timing)\n"
+               "  -cpu_only                   host side only: CPU line and the lists checked against the dense product\n");
         return 0;
     }
     const int M = (int)f.M, K = (int)f.K, N = (int)f.N, S = (int)f.S;
@@ -211,14 +349,11 @@ int main(int argc, char **argv)
     if (any) {
         pos.resize((size_t)N * (size_t)std::max(S / 2, 0));
         neg.resize(pos.size());
-        if ((f.i2s || f.check) && K > 0 && N > 0) dense.resize((size_t)K * N);
+        if ((f.i2s || f.cpu_only) && K > 0 && N > 0) dense.resize((size_t)K * N);
         CHECK_SPTMM(sptmm_generate_ternary(K, N, S, dense.empty() ? nullptr : dense.data(), pos.data(), neg.data()));
         if (f.row_split3_small && !sptmm_pack_u16_bytes(N, S, (int)f.row_split3_small)) strict_fail("Wrong split size");
         if (f.row_split_delta2 && !sptmm_pack_delta_bytes(N, S, (int)f.row_split_delta2, 8)) strict_fail("Wrong split size");
     }
-
-    sptmm_devinfo dev;
-    CHECK_SPTMM(sptmm_device_init(0, &dev));
 
     // activations (make_X, main.cu:784-797; seeded here)
     const uint32_t seed = f.seed ? (uint32_t)f.seed : (0xC0FFEEu ^ (uint32_t)M);
@@ -234,19 +369,90 @@ int main(int argc, char **argv)
         else
             for (size_t i = 0; i < xcount; ++i) ((uint16_t *)xhost.data())[i] = float_to_half(xf[i]);
     }
+
+    // The host's own result: the reference kernel's gather-sum over the lists this process holds (exact int32 for int8
+    // rows, double for float rows) -- what every device result below is compared with -- timed on one thread and on
+    // every core this process may use.
+    const int cores = affinity_cores(), half = S / 2;
+    std::vector<int32_t> host_i;
+    std::vector<double> host_f;
+    auto host_sum = [&](int c0, int c1) {  // columns [c0, c1)
+        if (act == 0)
+            host_gather_columns((const int8_t *)xhost.data(), M, K, N, half, pos.data(), neg.data(), c0, c1, host_i.data(), [](int8_t v) { return (int)v; });
+        else if (act == 1)
+            host_gather_columns((const uint16_t *)xhost.data(), M, K, N, half, pos.data(), neg.data(), c0, c1, host_f.data(),
+                                [](uint16_t v) { return (double)half_to_float(v); });
+        else
+            host_gather_columns((const float *)xhost.data(), M, K, N, half, pos.data(), neg.data(), c0, c1, host_f.data(), [](float v) { return (double)v; });
+    };
+    std::string cpu_line;
+    if (any && (f.check || f.cpu || f.cpu_only)) {
+        (act == 0 ? host_i.resize((size_t)M * N) : host_f.resize((size_t)M * N));
+        over_columns(N, cores, host_sum);
+        if (f.cpu || f.cpu_only) {
+            // steady clock, 3 warm-ups, median and minimum of up to 50 repetitions (at least 3; about a second per thread
+            // count), columns split statically over threads that live for the whole loop
+            auto time_it = [&](int threads, double *median, double *best, int *reps) {
+                std::vector<double> t = timed_over_columns(N, threads, 50, 1.0, host_sum);
+                std::sort(t.begin(), t.end());
+                *median = t[t.size() / 2], *best = t[0], *reps = (int)t.size();
+            };
+            double med_n = 0, min_n = 0, med_1 = 0, min_1 = 0;
+            int reps_n = 0, reps_1 = 0;
+            time_it(cores, &med_n, &min_n, &reps_n);
+            time_it(1, &med_1, &min_1, &reps_1);
+            const double bytes = 2.0 * S * N + (double)M * K * esz + 4.0 * M * N;
+            char buf[512];
+            snprintf(buf, sizeof buf,
+                     "# cpu: us/call threads=%d median=%.1f min=%.1f reps=%d (%.1f GB/s); threads=1 median=%.1f min=%.1f reps=%d (host "
+                     "gather-sum over the u16 lists, main.cu:577-593)",
+                     cores, med_n, min_n, reps_n, bytes / med_n / 1e3, med_1, min_1, reps_1);
+            cpu_line = buf;
+        }
+    }
+
+    auto banner = [&] {
+        std::cout << "make_X done" << std::endl;
+        printf("Compiled on %s at %s\n", __DATE__, __TIME__);
+        std::cout << "Start: "
+                  << "M=" << f.M << " K=" << f.K << " N=" << f.N << " ITER=" << f.iter << " S=" << f.S << " ("
+                  << (100.0 - 100.0 * ((float)f.S / (float)f.K)) << "% Sparsity)"
+                  << " L=" << f.L << " B=" << 8 << " X_MAJOR=ROW W_MAJOR=COL C_MAJOR=ROW" << std::endl;
+    };
+    if (f.cpu_only) {
+        // no device: the CPU line, and the lists' gather-sum against the dense product of the same matrix
+        banner();
+        if (!any) strict_fail("cpu_only needs a method (-row_split3_small, -row_split_delta2 or -i2s)");
+        bool pass;
+        double worst = 0;
+        if (act == 0) {
+            std::vector<int32_t> d((size_t)M * N);
+            host_dense_product((const int8_t *)xhost.data(), M, K, N, dense.data(), cores, d.data(), [](int8_t v) { return (int)v; });
+            pass = d == host_i;
+        } else {
+            std::vector<double> d((size_t)M * N);
+            if (act == 1)
+                host_dense_product((const uint16_t *)xhost.data(), M, K, N, dense.data(), cores, d.data(), [](uint16_t v) { return (double)half_to_float(v); });
+            else
+                host_dense_product((const float *)xhost.data(), M, K, N, dense.data(), cores, d.data(), [](float v) { return (double)v; });
+            for (size_t j = 0; j < d.size(); ++j)
+                worst = std::max(worst, std::fabs(d[j] - host_f[j]) / std::max(std::fabs(d[j]), std::sqrt((double)S)));
+            pass = worst <= 1e-9;
+        }
+        printf("%s\n", cpu_line.c_str());
+        printf("# check=%s (host gather-sum == host dense product; no device used)\n", pass ? "PASS" : "FAIL");
+        return pass ? 0 : 2;
+    }
+
+    sptmm_devinfo dev;
+    CHECK_SPTMM(sptmm_device_init(0, &dev));
     void *x_d = nullptr, *c_d = nullptr, *stream = nullptr;
     CHECK_SPTMM(sptmm_malloc(&x_d, xhost.size()));
     CHECK_SPTMM(sptmm_memcpy_h2d(x_d, xhost.data(), xhost.size()));
-    std::cout << "make_X done" << std::endl;
     CHECK_SPTMM(sptmm_malloc(&c_d, sizeof(int) * (size_t)M * N));
     CHECK_SPTMM(sptmm_memset(c_d, 0, sizeof(int) * (size_t)M * N));
     CHECK_SPTMM(sptmm_stream_create(&stream));
-
-    printf("Compiled on %s at %s\n", __DATE__, __TIME__);
-    std::cout << "Start: "
-              << "M=" << f.M << " K=" << f.K << " N=" << f.N << " ITER=" << f.iter << " S=" << f.S << " ("
-              << (100.0 - 100.0 * ((float)f.S / (float)f.K)) << "% Sparsity)"
-              << " L=" << f.L << " B=" << 8 << " X_MAJOR=ROW W_MAJOR=COL C_MAJOR=ROW" << std::endl;
+    banner();
 
     if (f.cu_blas) strict_fail("Wrong layout");  // main.cu:843: the row/col/row build refuses cuBLAS
 
@@ -329,37 +535,26 @@ int main(int argc, char **argv)
     }
 
     int status = 0;
+    if (!cpu_line.empty()) printf("%s\n", cpu_line.c_str());
     if (any && f.check) {
-        // the encodings are independent: make sure at least two of them have run, then compare all
-        if (done.size() < 2) {
-            sptmm_weights *w = nullptr;
-            if (act == 0 && !f.i2s) {
-                CHECK_SPTMM(sptmm_weights_upload_i2s(dense.data(), K, N, &w));
-                run("i2s(check)", w, false);
-            } else if (!f.row_split3_small && (S / 2) % 32 == 0) {
-                CHECK_SPTMM(sptmm_weights_upload_u16(pos.data(), neg.data(), K, N, S, 32, &w));
-                run("sptmm(check)", w, false);
-            } else if ((S / 2) % 8 == 0) {
-                CHECK_SPTMM(sptmm_weights_upload_delta(pos.data(), neg.data(), K, N, S, 8, &w));
-                run("sptmm-delta(check)", w, false);
-            }
-        }
-        bool pass = done.size() >= 2;
+        // every method's device output against the host gather-sum: bit-exact for int8 rows, within 1e-3 of
+        // max(|ref|, sqrt(S)) for float rows (fp32 sums on the device, double on the host)
+        bool pass = !done.empty();
         double worst = 0;
-        for (size_t i = 1; i < done.size(); ++i) {
+        for (const Method &m : done) {
             if (act == 0) {
-                pass &= done[i].result == done[0].result;
+                pass &= memcmp(m.result.data(), host_i.data(), m.result.size()) == 0;
             } else {
-                const float *a = (const float *)done[0].result.data(), *b = (const float *)done[i].result.data();
+                const float *g = (const float *)m.result.data();
                 for (size_t j = 0; j < (size_t)M * N; ++j) {
-                    double scale = std::max<double>(std::fabs(a[j]), std::sqrt((double)S));
-                    worst = std::max(worst, std::fabs((double)a[j] - b[j]) / scale);
+                    const double scale = std::max<double>(std::fabs(host_f[j]), std::sqrt((double)S));
+                    worst = std::max(worst, std::fabs((double)g[j] - host_f[j]) / scale);
                 }
                 pass &= worst <= 1e-3;
             }
         }
         printf("# check=%s (", pass ? "PASS" : "FAIL");
-        for (size_t i = 0; i < done.size(); ++i) printf("%s%s", i ? (act == 0 ? " == " : " ~ ") : "", done[i].label);
+        for (size_t i = 0; i < done.size(); ++i) printf("%s%s %s host", i ? "; " : "", done[i].label, act == 0 ? "==" : "~");
         if (act != 0) printf("; max rel diff %.2e", worst);
         printf(")\n");
         if (!pass) status = 2;

@@ -64,6 +64,45 @@ def test_help_lists_reference_flags():
         assert flag in r.stdout
 
 
+CPU_LINE = re.compile(r"^# cpu: us/call threads=(\d+) median=([0-9.]+) min=([0-9.]+) reps=(\d+) \(([0-9.]+) GB/s\); "
+                      r"threads=1 median=([0-9.]+) min=([0-9.]+) reps=(\d+) ")
+
+
+def check_cpu_line(out):
+    """`# cpu:` names the cores the process may use (its affinity mask) and gives median and minimum of at least 3 timed calls,
+    for all of them and for one thread."""
+    lines = [l for l in out.splitlines() if l.startswith("# cpu:")]
+    assert len(lines) == 1, out
+    m = CPU_LINE.match(lines[0])
+    assert m, lines[0]
+    assert int(m.group(1)) == len(os.sched_getaffinity(0))
+    assert float(m.group(3)) <= float(m.group(2)) and float(m.group(7)) <= float(m.group(6))
+    assert int(m.group(4)) >= 3 and int(m.group(8)) >= 3 and float(m.group(3)) > 0
+
+
+@pytest.mark.parametrize("args", [
+    ["-row_split3_small", "32", "-M=1", "-K=6912", "-N=2560", "-S=4096"],       # the headline shape, int8 rows
+    ["-row_split_delta2", "16", "-M=3", "-K=512", "-N=48", "-S=96", "-act", "f16"],
+    ["-i2s", "-M=2", "-K=256", "-N=32", "-S=128", "-act=f32"],
+    ["-row_split3_small", "8"],                                                  # the reference's default shape (main.cu:43-47)
+])
+def test_cpu_only_needs_no_device_and_checks_the_lists_against_the_dense_product(args):
+    """-cpu_only: the host gather-sum over the lists (main.cu:577-593 on the host) is timed and compared with the plain
+    dense product of the same seeded matrix; nothing touches a device."""
+    r = rcr(*args, "-cpu_only")
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.strip().splitlines()
+    assert lines[0] == "make_X done" and lines[2].startswith("Start: M=")
+    check_cpu_line(r.stdout)
+    assert lines[-1] == "# check=PASS (host gather-sum == host dense product; no device used)"
+    assert not [l for l in lines[3:] if not l.startswith("#")]  # no ms-per-call line: nothing ran on a device
+
+
+def test_cpu_only_without_a_method_aborts():
+    r = rcr("-cpu_only", "-M=1", "-K=64", "-N=16", "-S=32")
+    assert r.returncode == -signal.SIGABRT and "needs a method" in r.stderr
+
+
 FLOAT = re.compile(r"^[0-9]+(\.[0-9]+)?(e-?[0-9]+)?$")
 
 
@@ -79,7 +118,11 @@ def check_output(out, n_methods, M, K, N, S, iters):
     bare = [l for l in lines[3:] if not l.startswith("#")]
     assert len(bare) == n_methods and all(FLOAT.match(b) for b in bare), bare
     assert all(0 < float(b) < 10 for b in bare)  # milliseconds per call
-    assert any(l.startswith("# check=PASS") for l in lines), out
+    checks = [l for l in lines if l.startswith("# check=")]
+    assert len(checks) == 1 and checks[0].startswith("# check=PASS ("), out
+    # every method that ran is compared with the host's own gather-sum, not with another device result
+    assert checks[0].count("== host") == n_methods, checks[0]
+    check_cpu_line(out)
 
 
 @pytest.mark.gpu
@@ -103,6 +146,8 @@ def test_readme_command_lines(args, n):
 def test_float_activations_and_cublas_refusal():
     r = rcr("-row_split3_small", "32", "-row_split_delta2", "32", "-M=1", "-K=6912", "-N=2560", "-S=4096",
             "-iter=50", "-act", "f16")
-    assert r.returncode == 0 and "# check=PASS" in r.stdout, r.stdout + r.stderr
+    assert r.returncode == 0 and "# check=PASS (sptmm ~ host; sptmm-delta ~ host; max rel diff" in r.stdout, r.stdout + r.stderr
+    r = rcr("-row_split3_small", "32", "-M=2", "-K=512", "-N=64", "-S=128", "-iter=20", "-nocpu")
+    assert r.returncode == 0 and "# cpu:" not in r.stdout and "# check=PASS (sptmm == host)" in r.stdout, r.stdout + r.stderr
     r = rcr("-cu_blas", "-M=1", "-K=6912", "-N=2560", "-S=4096")
     assert r.returncode == -signal.SIGABRT and "Wrong layout" in r.stderr  # main.cu:843 in the row/col/row build

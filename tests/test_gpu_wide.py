@@ -135,6 +135,33 @@ def test_non_finite_fp16_row_stays_in_its_row_and_columns(bad):
         w.free()
 
 
+@pytest.mark.parametrize("bad", [np.inf, np.nan])
+def test_non_finite_value_in_one_k_tile_only(bad):
+    """Two K-tiles (K = 13824 -> 2 x 6912) whose finiteness differs: the tile with the Inf / NaN is summed on the vector
+    unit, the other on the matrix unit, and the two write the same outputs from different lanes of the wavefront.  The
+    second tile's sums are added to what the first stored, whichever path each took."""
+    K, N = 13824, 320
+    W = sp.generate_ternary_iid(K, N, 33, 0.3, 0.3)
+    for kind in (sp.KIND_U16, sp.KIND_DELTA):
+        w = sp.Weights.upload_wide(W, kind, 32)
+        assert w.info["k_tile"] == 6912
+        for k in (5, 6911, 6912, 13823):  # first tile only, then second tile only
+            say("wide non-finite, one K-tile", kind, k, bad)
+            X = oracle.make_x_normal(k, 8, K, np.float16)
+            X[5, k] = bad
+            clean = X.copy()
+            clean[5, k] = 0
+            got = w.matmul(X)
+            away = W[:, k] == 0
+            assert 0 < away.sum() < N
+            rows = [0, 1, 2, 3, 4, 6, 7]
+            assert np.isfinite(got[rows]).all() and np.isfinite(got[5, away]).all()
+            check_fp(got[rows], clean[rows], W)
+            check_fp(got[5:6, away], clean[5:6], W[away])
+            assert (~np.isfinite(got[5, ~away])).all()
+        w.free()
+
+
 def test_refusals():
     K, N = 512, 48
     W = sp.generate_ternary_iid(K, N, 1, 0.3, 0.3)
@@ -149,5 +176,8 @@ def test_refusals():
     assert e.value.code == -2
     with pytest.raises(sp.SptmmError):
         sp.Weights.upload_wide(W, sp.KIND_I2S, 32)
+    with pytest.raises(sp.SptmmError) as e:
+        sp.Weights.upload_wide(W, sp.KIND_U16, 128)  # wide streams take split_k up to 64; an explicit larger one is refused, not clamped
+    assert e.value.code == -1
     for o in (w, xb, cb):
         o.free()
