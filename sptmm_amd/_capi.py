@@ -429,11 +429,14 @@ def measure_gemv(weights, act: int, X: "DeviceBuffer", M: int, Cout: "DeviceBuff
     return us.value
 
 
+def _steps(steps):
+    return (Step * len(steps))(*[Step(w.handle, x.ptr, c.ptr, m, act, stage) for w, x, c, m, act, stage in steps])
+
+
 def measure_sequence(steps, reps: int, mode: int, stream: "Stream") -> float:
     """Mean microseconds per pass over `steps` = [(weights, X buffer, C buffer, M, act, stage), ...] (see sptmm_measure_sequence)."""
-    arr = (Step * len(steps))(*[Step(w.handle, x.ptr, c.ptr, m, act, stage) for w, x, c, m, act, stage in steps])
     us = C.c_double()
-    _ck(lib().sptmm_measure_sequence(arr, len(steps), reps, mode, stream.handle, C.byref(us)))
+    _ck(lib().sptmm_measure_sequence(_steps(steps), len(steps), reps, mode, stream.handle, C.byref(us)))
     return us.value
 
 

@@ -113,15 +113,9 @@ int finish_upload(sptmm_weights *w, const std::vector<uint8_t> &host, sptmm_weig
     return SPTMM_OK;
 }
 
-int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *stream, ActType act, int batch = 0,
-                const void *const *bw = nullptr, const void *const *bx = nullptr, void *const *bc = nullptr, int quant = 0,
-                float w_scale = 1.f)
+// what the launchers need to know of one GEMV on `w`
+void fill_args(const sptmm_weights *w, const void *X, int M, void *C, GemvArgs *out)
 {
-    if (!w || !X || !C) return fail(SPTMM_ERR_INVALID, "null pointer");
-    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
-    int dev = -1;
-    HIP_TRY(hipGetDevice(&dev));
-    if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
     GemvArgs a{};
     a.w = w->dev;
     a.X = X;
@@ -147,6 +141,30 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     a.ragged = w->info.ragged;
     a.compute_units = w->compute_units;
     a.lds_limit = w->lds_limit;
+    // A ragged stream whose tasks all hold the same number of entries, and whose tile keeps no zero slots, is laid out
+    // behind its count table exactly like a stream of balanced lists (the packers share slot_offset()): it runs on the
+    // kernels for tasks of one length -- no table look-ups, straight-line bodies of the exact length (K=6912 N=2560, 864
+    // entries per list, 32 GEMVs per launch: 0.81 -> 0.75 us per GEMV).
+    if (!w->wide && a.ragged && a.n_min == a.n_max && !a.stones && w->info.kind != SPTMM_KIND_I2S) {
+        a.ragged = 0;
+        a.n_lane = a.n_max;
+        a.w = (const uint8_t *)w->dev + w->counts_bytes;
+        a.batch_w_skip = (size_t)w->counts_bytes;  // (the list launchers add it to every stream of a batch)
+    }
+    *out = a;
+}
+
+int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *stream, ActType act, int batch = 0,
+                const void *const *bw = nullptr, const void *const *bx = nullptr, void *const *bc = nullptr, int quant = 0,
+                float w_scale = 1.f)
+{
+    if (!w || !X || !C) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
+    GemvArgs a;
+    fill_args(w, X, M, C, &a);
     a.quant = quant;
     a.w_scale = w_scale;
     a.batch = batch;
@@ -156,16 +174,6 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     if (w->wide) {
         if (quant) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
         return launch_wide(a, w->wh, act, stream);
-    }
-    // A ragged stream whose tasks all hold the same number of entries, and whose tile keeps no zero slots, is laid out
-    // behind its count table exactly like a stream of balanced lists (the packers share slot_offset()): it runs on the
-    // kernels for tasks of one length -- no table look-ups, straight-line bodies of the exact length (K=6912 N=2560, 864
-    // entries per list, 32 GEMVs per launch: 0.81 -> 0.75 us per GEMV).
-    if (a.ragged && a.n_min == a.n_max && !a.stones && w->info.kind != SPTMM_KIND_I2S) {
-        a.ragged = 0;
-        a.n_lane = a.n_max;
-        a.w = (const uint8_t *)w->dev + w->counts_bytes;
-        a.batch_w_skip = (size_t)w->counts_bytes;  // (the list launchers add it to every stream of a batch)
     }
     switch (w->info.kind) {
     case SPTMM_KIND_U16: return launch_u16(a, act, stream);
@@ -189,6 +197,7 @@ int sptmm_device_init(int device, sptmm_devinfo *out)
         if (e != hipSuccess || count == 0) return fail(SPTMM_ERR_HIP, "no HIP device available (%s)", hipGetErrorString(e));
         if (device < 0 || device >= count) return fail(SPTMM_ERR_INVALID, "device %d out of range (have %d)", device, count);
         HIP_TRY(hipSetDevice(device));
+        tuning_reload();  // the launch-shape overrides of tuning runs: read here, never on a launch path
         if (out) {
             hipDeviceProp_t pr;
             HIP_TRY(hipGetDeviceProperties(&pr, device));

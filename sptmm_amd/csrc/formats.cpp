@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <array>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <exception>
 #include <thread>
@@ -13,6 +14,28 @@
 #include "internal.hpp"
 
 namespace sptmm {
+
+namespace {
+Tuning g_tuning;
+}
+const Tuning &tuning() { return g_tuning; }
+void tuning_reload()
+{
+    auto knob = [](const char *name, int otherwise) {
+        const char *v = getenv(name);
+        return v && *v ? atoi(v) : otherwise;
+    };
+    Tuning t;
+    t.waves_per_wg = knob("SPTMM_WAVES_PER_WG", 0);
+    t.wgs_per_cu = knob("SPTMM_WGS_PER_CU", 0);
+    t.tasks_per_wave = knob("SPTMM_TASKS_PER_WAVE", 0);
+    t.wide_waves = knob("SPTMM_WIDE_WAVES", 0);
+    t.i2s_waves = knob("SPTMM_I2S_WAVES", 0);
+    t.i2s_ct = knob("SPTMM_I2S_CT", 0);
+    t.i2s_mfma_from = knob("SPTMM_I2S_MFMA_FROM", 2);
+    g_tuning = t;
+}
+
 
 static thread_local char g_err[512] = "";
 

@@ -400,8 +400,7 @@ static int launch_i2s_mfma_t(const GemvArgs &a, hipStream_t st, int waves)
 
 static int launch_i2s_mfma(const GemvArgs &a, hipStream_t st)
 {
-    static const int tune_waves = getenv("SPTMM_I2S_WAVES") ? atoi(getenv("SPTMM_I2S_WAVES")) : 0;
-    static const int tune_ct = getenv("SPTMM_I2S_CT") ? atoi(getenv("SPTMM_I2S_CT")) : 0;
+    const int tune_waves = tuning().i2s_waves, tune_ct = tuning().i2s_ct;
     const int rounds = i2s_padded_k(a.K) / 256, groups = a.N / 16;
     const int rows = a.M < 16 ? a.M : 16, xj = (rows + 3) / 4;  // loads of X rows per round: four rows each
     // Column tiles per wavefront and wavefronts per workgroup, measured on MI355X (K=6912 N=2560 and K=13824
@@ -445,7 +444,7 @@ int launch_i2s(const GemvArgs &a, void *stream)
     hipStream_t st = (hipStream_t)stream;
     // One activation row launched alone stays on the vector unit (dot4 on the codes as they are); with more
     // rows, or many GEMVs per launch, the matrix-unit kernel is ahead (M=4: 5.0 -> 3.5 us alone, 1.8 -> 0.8 us batched).
-    static const int mfma_from = getenv("SPTMM_I2S_MFMA_FROM") ? atoi(getenv("SPTMM_I2S_MFMA_FROM")) : 2;
+    const int mfma_from = tuning().i2s_mfma_from;
     if (a.M >= mfma_from || a.batch >= 4) return launch_i2s_mfma(a, st);
     if ((size_t)Kp + extra > (size_t)a.lds_limit) return launch_i2s_mfma(a, st);  // (K beyond the one-row LDS tile)
     return launch_i2s_t<1>(a, st, waves);

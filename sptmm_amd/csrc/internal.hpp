@@ -178,6 +178,20 @@ struct GemvArgs {
 };
 enum ActType { ACT_I8 = 0, ACT_F16 = 1, ACT_F32 = 2 };
 
+// Launch-shape overrides for tuning runs (0 = the launcher's own choice).  Filled from the environment by
+// sptmm_device_init -- once per call of it, never on a launch path -- and by nothing else.
+struct Tuning {
+    int waves_per_wg = 0;    // SPTMM_WAVES_PER_WG: wavefronts per workgroup of the list kernels
+    int wgs_per_cu = 0;      // SPTMM_WGS_PER_CU: workgroups per compute unit of a lone list launch
+    int tasks_per_wave = 0;  // SPTMM_TASKS_PER_WAVE: tasks per wavefront of a batched list launch
+    int wide_waves = 0;      // SPTMM_WIDE_WAVES: wavefronts per workgroup of the wide kernels
+    int i2s_waves = 0;       // SPTMM_I2S_WAVES
+    int i2s_ct = 0;          // SPTMM_I2S_CT: column tiles per wavefront of the i2s matrix-unit kernel
+    int i2s_mfma_from = 2;   // SPTMM_I2S_MFMA_FROM: rows from which a lone i2s launch takes the matrix-unit kernel
+};
+const Tuning &tuning();
+void tuning_reload();  // reads the environment (formats.cpp)
+
 int launch_u16(const GemvArgs &a, ActType act, void *stream);
 int launch_u16_scaled(const GemvArgs &a, ActType act, void *stream);   // lists_u16_scaled.hip
 int launch_u16_plain(const GemvArgs &a, ActType act, void *stream);    // lists_u16_plain.hip

@@ -1192,12 +1192,8 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // tiles take.  Measured on MI355X, K=2560 N=13824 split_k=32: one workgroup per CU 11.4 us,
     // two 6.3 us; the headline shape has 5 tasks per CU and stays at one workgroup of 5.
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
-    // launch-shape overrides for tuning runs; read once, or at every launch when SPTMM_TUNE_LIVE is set
-    auto knob = [](const char *name) { const char *v = getenv(name); return v ? atoi(v) : 0; };
-    static const bool tune_live = getenv("SPTMM_TUNE_LIVE") != nullptr;
-    static const int wpb0 = knob("SPTMM_WAVES_PER_WG"), wgs0 = knob("SPTMM_WGS_PER_CU"), tpw0 = knob("SPTMM_TASKS_PER_WAVE");
-    const int tune_wpb = tune_live ? knob("SPTMM_WAVES_PER_WG") : wpb0, tune_wgs = tune_live ? knob("SPTMM_WGS_PER_CU") : wgs0,
-              tune_tpw = tune_live ? knob("SPTMM_TASKS_PER_WAVE") : tpw0;
+    // launch-shape overrides for tuning runs (the environment as sptmm_device_init last read it)
+    const int tune_wpb = tuning().waves_per_wg, tune_wgs = tuning().wgs_per_cu, tune_tpw = tuning().tasks_per_wave;
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(lists_tile_rows(a) + 64) * SLOT;
     // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better

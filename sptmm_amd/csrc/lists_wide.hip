@@ -381,7 +381,7 @@ template <typename Act, int MODE, int RING, int MAXW>
 static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
 {
     constexpr int ROWS = WideSums<Act>::ROWS;
-    static const int tune_wpb = getenv("SPTMM_WIDE_WAVES") ? atoi(getenv("SPTMM_WIDE_WAVES")) : 0;
+    const int tune_wpb = tuning().wide_waves;
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
     const size_t lds = (size_t)(h.k_tile + 64) * 16 + 64;
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "the stream's K-tile of %d rows needs %zu bytes of LDS, the device grants %d", h.k_tile, lds, a.lds_limit);
