@@ -29,6 +29,7 @@ void tuning_reload()
     t.waves_per_wg = knob("SPTMM_WAVES_PER_WG", 0);
     t.wgs_per_cu = knob("SPTMM_WGS_PER_CU", 0);
     t.tasks_per_wave = knob("SPTMM_TASKS_PER_WAVE", 0);
+    t.share_log = knob("SPTMM_SHARE_LOG", 0);
     t.wide_waves = knob("SPTMM_WIDE_WAVES", 0);
     t.i2s_waves = knob("SPTMM_I2S_WAVES", 0);
     t.i2s_ct = knob("SPTMM_I2S_CT", 0);

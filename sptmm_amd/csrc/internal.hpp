@@ -188,6 +188,7 @@ struct Tuning {
     int i2s_waves = 0;       // SPTMM_I2S_WAVES
     int i2s_ct = 0;          // SPTMM_I2S_CT: column tiles per wavefront of the i2s matrix-unit kernel
     int i2s_mfma_from = 2;   // SPTMM_I2S_MFMA_FROM: rows from which a lone i2s launch takes the matrix-unit kernel
+    int share_log = 0;       // SPTMM_SHARE_LOG: a lone GEMV (one int8 row, u16 lists) gives each task 1 << this many wavefronts
 };
 const Tuning &tuning();
 void tuning_reload();  // reads the environment (formats.cpp)

@@ -700,9 +700,14 @@ struct ListsBody {
     // (so every wait on the stream is for one round only).  RF == 0: any number
     // of rounds, through a ring of RING rounds in flight.  RF == -1: no full round at all
     // (ragged: up to XMAX), only the tail.
-    template <int RF>
+    // SL > 0 (u16 lists, one int8 row, straight-line bodies): 1 << SL wavefronts of a workgroup share a task -- wavefront
+    // j of them takes the rounds j, j + (1 << SL), ... (RF counts the rounds of ONE wavefront), the first one the tail as
+    // well, and their per-column sums meet in LDS.  The launch then has 1 << SL times the wavefronts, each with that
+    // fraction of the gathers left to do once the last bytes of its rounds have arrived.
+    template <int RF, int SL = 0>
     static __device__ __forceinline__ void run(const ListParams &p, unsigned char *smem)
     {
+        static_assert(SL == 0 || (RF > 0 && MODE == 0 && !VAR && !QUANT && MT == 1 && sizeof(Act) == 1), "shared tasks: u16 lists, one int8 row");
         constexpr int NR = RF > 0 ? RF : 0;               // full rounds of the straight-line body (RF == -1: none, tails only)
         constexpr int NB = RF > 0 ? RF : RF == 0 ? RING : 1;
         // stepping-stone streams: item i (16 rows) goes to item i + i/6 of the tile, every seventh item stays zero
@@ -718,8 +723,9 @@ struct ListsBody {
         const unsigned short *const counts = reinterpret_cast<const unsigned short *>(p.w + RAGGED_PREAMBLE);
         // ragged: tasks differ in length; p.n_lane is the shortest, which is all the prologue may assume
         const int R0 = p.n_lane / E16;
-        int task = blockIdx.x * waves + wave;
-        const int task_step = p.grid_x * waves;
+        int task = (blockIdx.x * waves + wave) >> SL;
+        const int roff = wave & ((1 << SL) - 1);  // which of the task's wavefronts this one is
+        const int task_step = (p.grid_x * waves) >> SL;
         const Act *X = reinterpret_cast<const Act *>(p.X);
         typedef Quantiser<MT> Q;
         const unsigned short *Xq = reinterpret_cast<const unsigned short *>(p.X);
@@ -762,7 +768,7 @@ struct ListsBody {
             }
             if constexpr (RF > 0) {
 #pragma unroll
-                for (int i = 0; i < (RF < EARLY ? RF : EARLY); ++i) buf[i] = load_round(wp, i);
+                for (int i = 0; i < (RF < EARLY ? RF : EARLY); ++i) buf[i] = load_round(wp, (i << SL) + roff);
             } else if (RF == 0 && R0 > 0) {
 #pragma unroll
                 for (int i = 0; i < EARLY; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
@@ -825,7 +831,7 @@ struct ListsBody {
         if constexpr (RF > EARLY) {
             const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
 #pragma unroll
-            for (int i = EARLY; i < RF; ++i) buf[i] = load_round(wp, i);
+            for (int i = EARLY; i < RF; ++i) buf[i] = load_round(wp, (i << SL) + roff);
         } else if constexpr (RF == 0) {
             if (R0 > 0) {
                 const uint4 *wp = reinterpret_cast<const uint4 *>(tasks_base + (size_t)(task < p.tasks ? task : 0) * task_bytes + HDR) + lane;
@@ -906,7 +912,7 @@ struct ListsBody {
                 const int nxt = task + task_step;
                 n_ahead = counts[nxt < p.tasks ? nxt : 0];
             }
-            const int R = n_lane / E16, rem = n_lane - R * E16;
+            const int R = n_lane / E16, rem = SL > 0 && roff != 0 ? 0 : n_lane - R * E16;  // (R: rounds of the whole task)
             if (TWIN && plain) {
                 Plain pacc;
                 pacc.init();
@@ -919,7 +925,7 @@ struct ListsBody {
             if constexpr (RF != 0) {
                 if (!AHEAD && it > 0) {
 #pragma unroll
-                    for (int i = 0; i < NR; ++i) buf[i] = load_round(wp, i);
+                    for (int i = 0; i < NR; ++i) buf[i] = load_round(wp, (i << SL) + roff);
                 }
             } else {
                 // ring of RING rounds, loads clamped to the task's last round so that they stay unconditional
@@ -1105,11 +1111,24 @@ struct ListsBody {
                     part[wave * MT + lane] = t[0];
                 }
                 }  // two-tile epilogue
+            } else if constexpr (SL > 0) {
+                // the task's wavefronts leave their column sums side by side (8 columns per wavefront at most); the first adds them up
+                const int G = 64 >> p.logL;
+                A v = lanes_sum(acc.acc[0], p.logL);
+                if ((lane & ((1 << p.logL) - 1)) == 0) part[wave * 8 + (lane >> p.logL)] = v;
+                __syncthreads();
+                if (active && roff == 0 && lane < G) {
+                    A sum = (A)0;
+#pragma unroll
+                    for (int w = 0; w < (1 << SL); ++w) sum += part[(wave + w) * 8 + lane];
+                    C[(size_t)m0 * p.N + (task << (6 - p.logL)) + lane] = sum;
+                }
+                if (it + 1 < p.iters) __syncthreads();  // (the next task's sums go to the same place)
             } else {
                 store_lane_sums(p, acc.acc, part, back, active, task, lane, wave, m0);
             }
             }  // matrix-unit / plain sums
-            if (p.W != 1) {
+            if (SL == 0 && p.W != 1) {
                 // second pass: the W wavefronts of a column meet in a small LDS buffer
                 __syncthreads();
                 if (active && lane == 0 && (wave & (p.W - 1)) == 0) {
@@ -1143,6 +1162,14 @@ __global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, QUANT>())) list
 {
     extern __shared__ __align__(16) unsigned char smem[];
     ListsBody<Act, MT, MODE, PRE, VAR, QUANT, MERGED>::template run<RF>(p, smem);
+}
+
+// One int8 row on u16 lists with 1 << SL wavefronts per task (see ListsBody::run): up to 16 wavefronts per workgroup.
+template <bool PRE, int RF, int SL>
+__global__ void __launch_bounds__(1024) lists_kernel_shared(ListParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    ListsBody<int8_t, 1, 0, PRE, false, false, false>::template run<RF, SL>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -1360,6 +1387,62 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel launch");
 }
 
+// A lone GEMV of one int8 row on u16 lists whose tasks are 2, 4, 6 or 8 rounds long: 1 << SL wavefronts per task.
+// wpb wavefronts per workgroup (a multiple of 1 << SL), every workgroup resident.
+template <bool PRE, int RF, int SL>
+static int launch_lists_shared(const GemvArgs &a, int wpb, hipStream_t st)
+{
+    const size_t tile = (size_t)(a.K + 64) * 4, lds = tile + (size_t)wpb * 8 * 4;
+    if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
+    const int per_wg = wpb >> SL;  // tasks a workgroup holds at once
+    const int blocks = (a.tasks + per_wg - 1) / per_wg;
+    const int cus = a.compute_units > 0 ? a.compute_units : 256;
+    const int slots = cus * std::max(1, std::min(16 / wpb, (int)((size_t)a.lds_limit / lds)));
+    const int grid_x = blocks < slots ? blocks : slots;
+    const int iters = (blocks + grid_x - 1) / grid_x;
+    ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, a.n_lane, a.tasks, ilog2(a.L), a.W,
+                 0, 0, iters, 0, 1.f, 0, 64 * wpb, grid_x};
+    auto kern = lists_kernel_shared<PRE, RF, SL>;
+    static std::atomic<size_t> lds_granted{48 * 1024};
+    if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
+    hipLaunchKernelGGL(kern, dim3(grid_x), dim3(64 * wpb), lds, st, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel_shared launch");
+}
+
+// -> true and *rc when the launch went out with shared tasks
+template <typename Act, int MT, int MODE, bool PRE, bool VAR>
+static bool try_shared(const GemvArgs &a, hipStream_t st, int *rc)
+{
+    if constexpr (std::is_same<Act, int8_t>::value && MT == 1 && MODE == 0 && !VAR) {
+        if (a.batch || a.quant || a.W != 1 || a.M != 1) return false;
+        const int rounds = a.n_lane / 8, cus = a.compute_units > 0 ? a.compute_units : 256;
+        int sl = tuning().share_log, wpb = tuning().waves_per_wg;
+        if (sl < 0 || rounds < 2 || rounds > 8) return false;
+        if (sl == 0) {
+            // two wavefronts per task where the doubled launch is at most ten wavefronts per compute unit, in workgroups that
+            // hold a compute unit's share of the tasks.  One GEMV per launch, HBM-cold, without -> with (K=6912 N=2560):
+            // S=4096 split_k 32 (1280 tasks of 8 rounds) 5.62 -> 5.37 us, S=4160 5.87 -> 5.63, S=2048 split_k 16 (640 tasks
+            // of 8 rounds) 4.87 -> 3.88, S=1024 (4 rounds) 3.70 -> 3.12; K=2560 N=2560 S=1536 3.53 -> 3.51; beyond ten
+            // wavefronts per compute unit nothing (K=2560 N=6912, 1728 tasks: 5.39 -> 5.43), four wavefronts per task lose
+            // (headline 6.3-7.4 us).
+            if (rounds % 2 || 2 * (long)a.tasks > 10L * cus) return false;
+            sl = 1;
+            if (wpb <= 0) wpb = std::max(4, (int)((2L * a.tasks + cus - 1) / cus + 1) / 2 * 2);
+        }
+        if (rounds % (1 << sl)) return false;
+        if (wpb <= 0) wpb = 8;
+        if (wpb > 16 || wpb % (1 << sl)) return false;
+        const int rf = rounds >> sl;
+#define SHARED_CASE(RF_, SL_) \
+    if (rf == RF_ && sl == SL_) return *rc = launch_lists_shared<PRE, RF_, SL_>(a, wpb, st), true
+        SHARED_CASE(4, 1); SHARED_CASE(3, 1); SHARED_CASE(2, 1); SHARED_CASE(1, 1);
+        SHARED_CASE(2, 2); SHARED_CASE(1, 2);
+#undef SHARED_CASE
+    }
+    return false;
+}
+
 // Straight-line bodies exist for tasks
 // with 1, 2, 3, 4, 6 or 8 full rounds (ragged streams: for the shortest
 // task, when the longest has at most XMAX more); everything else takes the ring.
@@ -1377,6 +1460,8 @@ template <typename Act, int MT, int MODE, bool PRE, bool VAR>
 static int launch_lists_t(const GemvArgs &a, hipStream_t st)
 {
     {
+        int rc = SPTMM_OK;
+        if (try_shared<Act, MT, MODE, PRE, VAR>(a, st, &rc)) return rc;
         constexpr int E16 = 16 / Flavour<MODE>::ESZ;
         int rf = (VAR ? a.n_min : a.n_lane) / E16;
         if constexpr (VAR) {
