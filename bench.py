@@ -189,6 +189,35 @@ def layer_sequence(sp, st, checks, reps):
                         "us per layer between two HIP events around `reps` passes (sptmm_measure_sequence)"}
 
 
+def plans_leg(sp, n_shapes=12):
+    """The launch-shape model against a bounded on-device search (sptmm_weights_tune), over seeded random shapes the model
+    was never fitted on: K and N multiples of 256, 8-60 % nonzeros, both list encodings, a lone GEMV, a batched launch of 16
+    GEMVs, and one of 16 four-row products.  Microseconds per GEMV, HBM-cold, with the model's shape and with the best plan found."""
+    import numpy as np
+
+    rng = np.random.default_rng(20250)
+    rows = []
+    for i in range(n_shapes):
+        k_rows = int(rng.integers(4, 55)) * 256
+        n_cols = int(rng.integers(1, 33)) * 256
+        s_nz = max(32, int(k_rows * rng.uniform(0.08, 0.6)) // 32 * 32)
+        Wm, p, n = sp.generate_ternary(k_rows, n_cols, s_nz)
+        for enc in ("u16", "delta"):
+            for m, batch in ((1, 0), (1, 16), (4, 16)):
+                w = sp.Weights.upload_u16(p, n, k_rows, 0) if enc == "u16" else sp.Weights.upload_delta(p, n, k_rows, 0, rows=m)
+                us_model, us_best, plan = w.tune(m, batch)
+                rows.append({"K": k_rows, "N": n_cols, "S": s_nz, "enc": enc, "M": m, "gemvs_per_launch": batch or 1, "split_k": w.info["split_k"],
+                             "model_us": round(us_model, 3), "best_plan_us": round(us_best, 3), "model_over_best": round(us_model / us_best, 3),
+                             "plan": {k: v for k, v in plan.items() if v}})
+                w.free()
+    worst = max(rows, key=lambda r: r["model_over_best"])
+    over = [r for r in rows if r["model_over_best"] > 1.10]
+    return {"rows": rows, "summary": {"cases": len(rows), "model_more_than_10pct_behind_best_plan": len(over),
+                                      "worst_model_over_best": worst["model_over_best"],
+                                      "worst_case": {k: worst[k] for k in ("K", "N", "S", "enc", "M", "gemvs_per_launch")},
+                                      "median_model_over_best": round(float(np.median([r["model_over_best"] for r in rows])), 3)}}
+
+
 def run(argv=None):
     """-> the full result: the contract keys plus every leg's table."""
     ap = argparse.ArgumentParser()
@@ -199,13 +228,14 @@ def run(argv=None):
     ap.add_argument("--reps", type=int, default=0,
                     help="launches per timed loop of the legs (0: 1500, the headline shape's other encodings 4096); counter "
                          "runs under a profiler, where every launch is serialised, use a few dozen")
-    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,layer,cfg4,density",
+    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,layer,cfg4,density,plans",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, sync-each-call, four streams), "
                          "others (delta and i2s encodings at the headline shape), cfg1 (the same matrix at M=4), cfg2 (gap "
                          "stream with fp16 rows), cfg3 (decoder-layer shapes, M=1 and 4), cfg4 (K=13824 N=5120, M=1/8/16), "
                          "layer (config 3 as a sequence: the decoder layer's 7 projections, or 4 with q+k+v and gate+up fused, "
                          "issued in order / as a HIP graph, rotating over enough layers to stay HBM-cold), "
                          "density (the headline shape at 3.7-25 % nonzeros against i2s), "
+                         "plans (the launch-shape model against sptmm_weights_tune over random shapes), "
                          "copy (4 launches of a 1 GiB copy kernel, for counter calibration), ceiling (a pure streaming "
                          "read of as many bytes as one step moves); profiling runs use --legs none or one leg")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
@@ -272,19 +302,21 @@ def run(argv=None):
         rows over zero slots of the tile instead of widening every gap to 16 bits."""
         Wm, p, n = lists if lists is not None else sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)
         rows = []
-        # gap streams are packed for the number of activation rows they will meet: the GEMV stream (rows = 1) or the plain one
-        makers = (("u16", lambda m: sp.Weights.upload_u16(p, n, k_rows, split)),
+        # streams are built for the number of activation rows they will meet (the _rows upload calls): the gap stream for
+        # GEMVs at M = 1, wide streams -- the lists read once for up to 16 rows -- beyond 8 rows
+        makers = (("u16", lambda m: sp.Weights.upload_u16(p, n, k_rows, split if m <= 8 or split <= 64 else 0, rows=m)),
                   ("delta", (lambda m: sp.Weights.upload_dense(Wm, sp.KIND_DELTA, split, rows=m)) if from_dense else
                             (lambda m: sp.Weights.upload_delta(p, n, k_rows, split, rows=m))),
                   ("i2s", lambda m: sp.Weights.upload_i2s(Wm)))
+        built_for = lambda enc, m: 0 if enc == "i2s" else 16 if m > 8 else 1 if (m == 1 and enc == "delta") else 4
         refs = {}
         for enc, mk in makers:
-            w = None
+            w, have = None, None
             for m in ms:
-                if w is None or (enc == "delta" and (m == 1) != (w.info["row_bytes"] == 1)):
+                if w is None or built_for(enc, m) != have:
                     if w is not None:
                         w.free()
-                    w = mk(m)
+                    w, have = mk(m), built_for(enc, m)
                 Xm = sp.make_x_i8(0xC0FFEE ^ m, m, k_rows)
                 got = w.matmul(Xm)
                 if m not in refs:
@@ -292,7 +324,7 @@ def run(argv=None):
                     checks.append(("%s M=%d" % (label, m), Xm, p, n, got, s_nz))
                 r = {"shape": label, "K": k_rows, "N": n_cols, "S": s_nz, "M": m, "enc": enc, "split_k": w.info["split_k"],
                      "row_bytes": w.info["row_bytes"], "delta_bits": w.info["delta_bits"], "zero_slot_detours": w.info["stones"],
-                     "bit_exact_across_encodings": bool((got == refs[m]).all())}
+                     "k_tile": w.info["k_tile"], "bit_exact_across_encodings": bool((got == refs[m]).all())}
                 r.update(time_encoding(w, 0, Xm, m, n_cols, k_rows))
                 rows.append(r)
             w.free()
@@ -415,15 +447,17 @@ def run(argv=None):
         configs["cfg3_layer"] = {"shapes": rows, "summed_layer": sums}
     if "cfg4" in legs:
         rows = run_matrix(*LARGE, (1, 8, 16))
-        # the same matrix as wide streams (K-tiled, 16-row tiles): the lists read once at M = 16, where the ordinary
-        # streams take two passes of eight rows because a 16-row tile of K = 13824 does not fit the LDS
+        # M = 16 above ran on wide streams (K-tiled, 16-row tiles: the lists read once), which is what an upload that declares
+        # 16 rows builds.  For comparison the ordinary streams at M = 16: two passes of eight rows, because a 16-row tile of
+        # K = 13824 does not fit the LDS.
         name, k_rows, n_cols, s_nz = LARGE
-        Wl = sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)[0]
+        Wl, pl, nl = sp.generate_ternary(k_rows, n_cols, s_nz, dense=True)
         X16 = sp.make_x_i8(0xC0FFEE ^ 16, 16, k_rows)
         ref16 = next(g for lab, xx, _, _, g, _ in checks if lab == "large M=16")
-        for enc, kind in (("wide u16", sp.KIND_U16), ("wide delta", sp.KIND_DELTA)):
-            ww = sp.Weights.upload_wide(Wl, kind, 32)
-            r = {"shape": name, "K": k_rows, "N": n_cols, "S": s_nz, "M": 16, "enc": enc, "split_k": 32, "k_tile": ww.info["k_tile"],
+        for enc, mk in (("u16, ordinary stream in two passes", lambda: sp.Weights.upload_u16(pl, nl, k_rows, 0)),
+                        ("delta, ordinary stream in two passes", lambda: sp.Weights.upload_delta(pl, nl, k_rows, 0))):
+            ww = mk()
+            r = {"shape": name, "K": k_rows, "N": n_cols, "S": s_nz, "M": 16, "enc": enc, "split_k": ww.info["split_k"], "k_tile": ww.info["k_tile"],
                  "bit_exact_across_encodings": bool((ww.matmul(X16) == ref16).all())}
             r.update(time_encoding(ww, 0, X16, 16, n_cols, k_rows))
             rows.append(r)
@@ -452,6 +486,8 @@ def run(argv=None):
                           "lists_over_i2s": round(best["batched_us"] / i2s_us, 3)})
         wins = [c["density_pct"] for c in cross if c["lists_over_i2s"] < 1.0]
         density = {"shapes": rows, "against_i2s": cross, "lists_beat_i2s_up_to_density_pct": max(wins) if wins else None}
+
+    plans = plans_leg(sp) if "plans" in legs else None
 
     gbps = nbytes / us_gemv / 1e3
     traffic, traffic_src = None, None
@@ -486,7 +522,7 @@ def run(argv=None):
             # at BASELINE's 59 % nonzeros the lists hold 4.7x (gap stream 2.4x) the bytes of i2s; they win where they are smaller
             "beats_i2s_batched_up_to_density_pct": density["lists_beat_i2s_up_to_density_pct"] if density else None,
         },
-        "single_launch": single, "other_encodings": others, "configs": configs, "layer_sequence": layer_seq, "density_sweep": density,
+        "single_launch": single, "other_encodings": others, "configs": configs, "layer_sequence": layer_seq, "density_sweep": density, "launch_plans": plans,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_src,
@@ -553,12 +589,14 @@ def final_line(full):
         summary["cfg3_layer_summed"] = {"M%d_%s" % (t["M"], t["enc"]): [t["batched_us"], t["batched_pct_roofline"], t["alone_cold_us"]]
                                         for t in cf["cfg3_layer"]["summed_layer"]}
     if "cfg4_large" in cf:
-        summary["cfg4_large"] = {"M%d_%s" % (r["M"], r["enc"].replace(" ", "_")): brief(r) for r in cf["cfg4_large"]}
+        summary["cfg4_large"] = {"M%d_%s" % (r["M"], r["enc"].split(",")[0] + ("_two_passes" if "," in r["enc"] else "")): brief(r) for r in cf["cfg4_large"]}
     if full.get("layer_sequence"):
         summary["layer_sequence"] = full["layer_sequence"]["summary"]
     dn = full.get("density_sweep")
     if dn:
         summary["density_lists_over_i2s"] = {str(c["density_pct"]): c["lists_over_i2s"] for c in dn["against_i2s"]}
+    if full.get("launch_plans"):
+        summary["launch_plans_model_vs_tuned"] = full["launch_plans"]["summary"]
     out["summary"] = summary
     out["detail_file"] = full.get("detail_file")
     return json.dumps(out, ensure_ascii=False, separators=(",", ":"))
@@ -575,7 +613,7 @@ def main():
                 json.dump(full, f, ensure_ascii=False, indent=1)
         except OSError as e:  # a read-only tree: the tables still go to stderr
             print("bench.py: cannot write %s: %s" % (path, e), file=sys.stderr)
-    for leg in ("single_launch", "other_encodings", "configs", "layer_sequence", "density_sweep"):
+    for leg in ("single_launch", "other_encodings", "configs", "layer_sequence", "density_sweep", "launch_plans"):
         if full.get(leg):
             print(json.dumps({leg: full[leg]}, ensure_ascii=False), file=sys.stderr)
     print(final_line(full), flush=True)

@@ -187,6 +187,11 @@ int sptmm_device_init(int device, sptmm_devinfo *out);
  * current device (ragged matrices: from the mean nonzeros per column). */
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
 int sptmm_weights_upload_delta(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out);
+/* The _rows forms say how many activation rows the calls on this stream will bring, and the stream is built for
+ * that: rows > 8 gives a WIDE stream (sptmm_weights_upload_wide: the lists read once for up to 16 int8 rows, where an
+ * ordinary stream serves such a call in passes of eight rows and reads the lists once per pass; info.k_tile != 0
+ * says so; u16: only for split_k <= 64 or 0); rows = 0: no preference.  Any stream still serves any M. */
+int sptmm_weights_upload_u16_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int rows, sptmm_weights **out);
 /* Gap stream scheduled for calls with `rows` activation rows (sptmm_pack_delta_rows): rows = 1 is
  * the stream for GEMVs (int8, M = 1); 0 = no preference (as sptmm_weights_upload_delta).
  * Byte gaps where every gap fits; else the smaller of 16-bit gaps and the 8-bit stream that
@@ -220,6 +225,29 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path);
 int sptmm_weights_load(const char *path, sptmm_weights **out);
 int sptmm_weights_info(const sptmm_weights *w, sptmm_winfo *out);
 size_t sptmm_weights_bytes(const sptmm_weights *w);
+
+/* Launch plans.  The shape of a launch (wavefronts per workgroup, workgroups per compute unit, tasks per wavefront, ...)
+ * comes from a model inside the library; a stream may carry its own choice per kind of call -- by activation rows
+ * (1, 2-4, 5-8, more) and by lone or batched launch -- which then replaces the model's for that stream.  Every field
+ * 0 = the model's choice; a value the kernels cannot take is ignored, never an error, and no plan changes a result.
+ * The reference fixes its launch shapes at compile time (grid and block per instantiation, main.cu:996-1455).
+ *   sptmm_weights_tune: a bounded search on the device -- a few dozen candidate plans, each timed over launches that
+ *   rotate over device copies of the stream (HBM-cold; `batch` = 0 times lone launches, else launches of `batch`
+ *   GEMVs; act as in sptmm_gemv_batched; int8, fp16 or fp32 rows of zeros) -- which stores the fastest as the stream's
+ *   plan for that kind of call and reports microseconds per GEMV under the model's shape and under the plan kept (the
+ *   model's shape is kept unless a candidate is at least 2 % faster).  Synchronous; allocates and frees its own buffers.
+ * Plans travel with sptmm_weights_save / _load and are copied by sptmm_weights_clone. */
+typedef struct sptmm_plan {
+    int waves_per_wg;    /* wavefronts per workgroup */
+    int wgs_per_cu;      /* workgroups per compute unit, lone list launches */
+    int tasks_per_wave;  /* tasks per wavefront, batched list launches */
+    int share_log;       /* lone GEMV of one int8 row on u16 lists: 1 << share_log wavefronts per task; -1: never shared */
+    int i2s_ct;          /* i2s: column tiles per wavefront (1, 2, 4, 8) */
+    int reserved[3];
+} sptmm_plan;
+int sptmm_weights_set_plan(sptmm_weights *w, int M, int batched, const sptmm_plan *plan);
+int sptmm_weights_get_plan(const sptmm_weights *w, int M, int batched, sptmm_plan *out);
+int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_model, double *us_tuned);
 
 /* C[M][N] = X[M][K] . W, X and C row-major device pointers (main.cu:575,592).
  * Asynchronous on `stream`.  The device that held the weights at upload must be

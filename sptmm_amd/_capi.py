@@ -11,7 +11,7 @@ __all__ = [
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
     "generate_ternary_iid", "dense_from_i2s_words", "choose_split_k", "wide_k_tile", "pack_wide", "unpack_wide",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
-    "device_sync", "Graph", "measure_gemv", "measure_sequence", "Step", "SEQ_MODES", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
+    "device_sync", "Graph", "measure_gemv", "measure_sequence", "Step", "SEQ_MODES", "PlanStruct", "gemv_i8_batched", "gemv_batched", "KIND_U16", "KIND_DELTA", "KIND_I2S", "EXPORTS",
 ]
 
 KIND_U16, KIND_DELTA, KIND_I2S = 1, 2, 3
@@ -29,7 +29,7 @@ EXPORTS = [
     "sptmm_unpack_ragged", "sptmm_generate_ternary_iid", "sptmm_dense_from_i2s_words", "sptmm_weights_upload_dense",
     "sptmm_choose_split_k", "sptmm_wide_k_tile", "sptmm_pack_wide_bytes", "sptmm_pack_wide", "sptmm_unpack_wide", "sptmm_weights_upload_wide",
     "sptmm_device_init",
-    "sptmm_weights_upload_u16", "sptmm_weights_upload_delta", "sptmm_weights_upload_delta_rows", "sptmm_weights_upload_dense_rows",
+    "sptmm_weights_upload_u16", "sptmm_weights_upload_u16_rows", "sptmm_weights_upload_delta", "sptmm_weights_upload_delta_rows", "sptmm_weights_upload_dense_rows",
     "sptmm_pack_delta_rows", "sptmm_pack_ragged_rows",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
@@ -38,7 +38,7 @@ EXPORTS = [
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
     "sptmm_graph_begin", "sptmm_graph_end", "sptmm_graph_launch", "sptmm_graph_destroy",
-    "sptmm_stream_wait_event", "sptmm_measure_sequence",
+    "sptmm_stream_wait_event", "sptmm_measure_sequence", "sptmm_weights_set_plan", "sptmm_weights_get_plan", "sptmm_weights_tune",
 ]
 
 
@@ -58,6 +58,13 @@ class WInfo(C.Structure):
     _fields_ = [("kind", C.c_int), ("K", C.c_int), ("N", C.c_int), ("S", C.c_int), ("split_k", C.c_int),
                 ("delta_bits", C.c_int), ("stream_bytes", C.c_uint64),
                 ("ragged", C.c_int), ("nnz", C.c_uint64), ("k_tile", C.c_int), ("row_bytes", C.c_int), ("stones", C.c_int)]
+
+
+class PlanStruct(C.Structure):
+    """sptmm_plan: the launch shape of one kind of call on one stream (0 = the library's model)."""
+    _fields_ = [("waves_per_wg", C.c_int), ("wgs_per_cu", C.c_int), ("tasks_per_wave", C.c_int), ("share_log", C.c_int), ("i2s_ct", C.c_int),
+                ("reserved", C.c_int * 3)]
+    NAMES = ("waves_per_wg", "wgs_per_cu", "tasks_per_wave", "share_log", "i2s_ct")
 
 
 class Step(C.Structure):
@@ -119,6 +126,9 @@ def lib() -> C.CDLL:
         L.sptmm_graph_launch.argtypes = [C.c_void_p, C.c_void_p]
         L.sptmm_graph_destroy.argtypes = [C.c_void_p]
         L.sptmm_event_elapsed_us.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]
+        L.sptmm_weights_set_plan.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(PlanStruct)]
+        L.sptmm_weights_get_plan.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(PlanStruct)]
+        L.sptmm_weights_tune.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
         L.sptmm_stream_wait_event.argtypes = [C.c_void_p, C.c_void_p]
         L.sptmm_measure_sequence.argtypes = [C.POINTER(Step), C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]
         _LIB = L
@@ -482,10 +492,11 @@ class Weights:
         self.handle = handle
 
     @classmethod
-    def upload_u16(cls, pos, neg, K, split_k) -> "Weights":
+    def upload_u16(cls, pos, neg, K, split_k, rows=0) -> "Weights":
+        """rows: activation rows per call the stream is built for (more than 8: a wide stream; 0: no preference)."""
         N, half = pos.shape
         h = C.c_void_p()
-        _ck(lib().sptmm_weights_upload_u16(_p(pos), _p(neg), K, N, 2 * half, split_k, C.byref(h)))
+        _ck(lib().sptmm_weights_upload_u16_rows(_p(pos), _p(neg), K, N, 2 * half, split_k, rows, C.byref(h)))
         return cls(h)
 
     @classmethod
@@ -542,6 +553,26 @@ class Weights:
     @property
     def nbytes(self) -> int:
         return int(lib().sptmm_weights_bytes(self.handle))
+
+    # launch plans (see sptmm_plan): the stream's own launch shape per kind of call, zeros = the library's model
+    def set_plan(self, M: int, batched: bool, **fields):
+        p = PlanStruct()
+        for k, v in fields.items():
+            assert k in PlanStruct.NAMES, k
+            setattr(p, k, int(v))
+        _ck(lib().sptmm_weights_set_plan(self.handle, M, int(bool(batched)), C.byref(p)))
+
+    def get_plan(self, M: int, batched: bool) -> dict:
+        p = PlanStruct()
+        _ck(lib().sptmm_weights_get_plan(self.handle, M, int(bool(batched)), C.byref(p)))
+        return {k: getattr(p, k) for k in PlanStruct.NAMES}
+
+    def tune(self, M: int, batch: int = 0, act: int = 0):
+        """Bounded on-device search for the launch shape of calls with M rows (batch = 0: lone launches, else launches of
+        `batch` GEMVs); the fastest plan is stored in the object.  -> (us per GEMV with the model's shape, with the plan kept, plan)."""
+        a, b = C.c_double(), C.c_double()
+        _ck(lib().sptmm_weights_tune(self.handle, M, batch, act, C.byref(a), C.byref(b)))
+        return a.value, b.value, self.get_plan(M, batch > 0)
 
     # raw launches on device buffers (asynchronous on `stream`)
     def gemv_i8(self, X: DeviceBuffer, M: int, Cout: DeviceBuffer, stream: Stream | None = None):

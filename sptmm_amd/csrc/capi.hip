@@ -27,9 +27,13 @@ struct sptmm_weights {
     bool stones = false;     // 8-bit gap stream of tile positions (zero slots behind every 96 rows of the tile)
     bool wide = false;    // wide stream (K-tiled, 16-byte slots): `wh` describes it
     WideHeader wh;
+    Plan plans[PLAN_SLOTS];  // the stream's own launch shapes, by kind of call (plan_slot); zeros: the launchers' model
 };
 
 namespace {
+
+int measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters, int mode, void *stream,
+                 double *us_per_call);
 
 int hip_fail(hipError_t e, const char *what)
 {
@@ -85,6 +89,27 @@ int resolve_split_dense(const int8_t *W, int K, int N, int kind, int *split_k)
     if (S < 512) S = 512;
     return resolve_split(kind, (N + 15) / 16 * 16, (int)S, split_k);
 }
+
+// balanced lists -> the dense matrix (column n at W + n*K); SPTMM_ERR_INVALID for a row index beyond K
+int dense_from_lists(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, std::vector<int8_t> *W)
+{
+    if (!pos || !neg) return fail(SPTMM_ERR_INVALID, "null pointer");
+    W->assign((size_t)K * N, 0);
+    for (int sign = 0; sign < 2; ++sign) {
+        const uint16_t *l = sign ? neg : pos;
+        for (int c = 0; c < N; ++c)
+            for (int i = 0; i < S / 2; ++i) {
+                const uint16_t r = l[(size_t)c * (S / 2) + i];
+                if (r >= K) return fail(SPTMM_ERR_INVALID, "row index %d out of range in column %d", (int)r, c);
+                (*W)[(size_t)c * K + r] = sign ? (int8_t)-1 : (int8_t)1;
+            }
+    }
+    return SPTMM_OK;
+}
+
+// Streams declared for more than eight activation rows per call are wide streams: the ordinary ones serve such calls
+// in passes of eight rows and read the lists once per pass.
+constexpr int ROWS_PER_PASS = 8;
 
 int finish_upload(sptmm_weights *w, const std::vector<uint8_t> &host, sptmm_weights **out)
 {
@@ -165,6 +190,15 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
     GemvArgs a;
     fill_args(w, X, M, C, &a);
+    {
+        // the stream's plan for this kind of call over the process-wide overrides over the launchers' model
+        const Plan &mine = w->plans[plan_slot(M, batch > 0)], &all = tuning().plan;
+        a.plan.waves_per_wg = mine.waves_per_wg ? mine.waves_per_wg : all.waves_per_wg;
+        a.plan.wgs_per_cu = mine.wgs_per_cu ? mine.wgs_per_cu : all.wgs_per_cu;
+        a.plan.tasks_per_wave = mine.tasks_per_wave ? mine.tasks_per_wave : all.tasks_per_wave;
+        a.plan.share_log = mine.share_log ? mine.share_log : all.share_log;
+        a.plan.i2s_ct = mine.i2s_ct ? mine.i2s_ct : all.i2s_ct;
+    }
     a.quant = quant;
     a.w_scale = w_scale;
     a.batch = batch;
@@ -217,9 +251,22 @@ int sptmm_device_init(int device, sptmm_devinfo *out)
 
 int sptmm_weights_upload_u16(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, sptmm_weights **out)
 {
+    return sptmm_weights_upload_u16_rows(pos, neg, K, N, S, split_k, 0, out);
+}
+
+int sptmm_weights_upload_u16_rows(const uint16_t *pos, const uint16_t *neg, int K, int N, int S, int split_k, int rows, sptmm_weights **out)
+{
     return guarded([&]() -> int {
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         if (int rc = check_shape(K, N, S)) return rc;
+        if (rows > ROWS_PER_PASS && (split_k == 0 || split_k <= 64)) {
+            std::vector<int8_t> W;
+            if (int rc = dense_from_lists(pos, neg, K, N, S, &W)) return rc;
+            if (int rc = sptmm_weights_upload_wide(W.data(), K, N, SPTMM_KIND_U16, split_k, out)) return rc;
+            (*out)->info.S = S;
+            return SPTMM_OK;
+        }
         if (int rc = resolve_split(SPTMM_KIND_U16, N, S, &split_k)) return rc;
         Geometry g;
         if (int rc = make_geometry(N, S, split_k, 256, &g)) return rc;
@@ -245,6 +292,13 @@ int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, in
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
         if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         if (int rc = check_shape(K, N, S)) return rc;
+        if (rows > ROWS_PER_PASS) {
+            std::vector<int8_t> W;
+            if (int rc = dense_from_lists(pos, neg, K, N, S, &W)) return rc;
+            if (int rc = sptmm_weights_upload_wide(W.data(), K, N, SPTMM_KIND_DELTA, split_k, out)) return rc;
+            (*out)->info.S = S;
+            return SPTMM_OK;
+        }
         if (int rc = resolve_split(SPTMM_KIND_DELTA, N, S, &split_k)) return rc;
         Geometry g;
         if (int rc = make_geometry(N, S, split_k, 64, &g)) return rc;
@@ -254,16 +308,8 @@ int sptmm_weights_upload_delta_rows(const uint16_t *pos, const uint16_t *neg, in
             // Some gap is too long for a byte (the reference narrows every gap to u8 unchecked, main.cu:376-394).  The
             // builder for arbitrary matrices can walk long gaps over zero slots of the tile; take its stream where
             // that is smaller than 16-bit gaps throughout.
-            std::vector<int8_t> W((size_t)K * N, 0);
-            for (int sign = 0; sign < 2; ++sign) {
-                const uint16_t *l = sign ? neg : pos;
-                for (int c = 0; c < N; ++c)
-                    for (int i = 0; i < S / 2; ++i) {
-                        const uint16_t r = l[(size_t)c * (S / 2) + i];
-                        if (r >= K) return fail(SPTMM_ERR_INVALID, "row index %d out of range in column %d", (int)r, c);
-                        W[(size_t)c * K + r] = sign ? (int8_t)-1 : (int8_t)1;
-                    }
-            }
+            std::vector<int8_t> W;
+            if (int rc = dense_from_lists(pos, neg, K, N, S, &W)) return rc;
             sptmm_weights *alt = nullptr;
             if (sptmm_weights_upload_dense_rows(W.data(), K, N, SPTMM_KIND_DELTA, split_k, rows, &alt) == SPTMM_OK) {
                 if (alt->info.delta_bits == 8) {
@@ -313,6 +359,7 @@ int sptmm_weights_upload_dense_rows(const int8_t *W, int K, int N, int kind, int
         if (!out) return fail(SPTMM_ERR_INVALID, "null pointer");
         if (rows < 0) return fail(SPTMM_ERR_INVALID, "rows must be 0 (any) or the activation rows per call");
         if (kind == SPTMM_KIND_I2S) return sptmm_weights_upload_i2s(W, K, N, out);
+        if (rows > ROWS_PER_PASS && (split_k == 0 || split_k <= 64)) return sptmm_weights_upload_wide(W, K, N, kind, split_k, out);
         if (int rc = resolve_split_dense(W, K, N, kind, &split_k)) return rc;
         int bits = 0, n_min = 0, n_max = 0;
         size_t read_bytes = 0;
@@ -350,8 +397,11 @@ int sptmm_weights_upload_wide(const int8_t *W, int K, int N, int kind, int split
         const int k_tile = sptmm_wide_k_tile(K, caps.lds);
         if (k_tile < 0) return k_tile;
         if (split_k > 64) return fail(SPTMM_ERR_INVALID, "wide streams take split_k 8, 16, 32 or 64 (or 0: the library's pick), not %d", split_k);
+        const bool pick = split_k == 0;
         if (int rc = resolve_split_dense(W, K, N, kind, &split_k)) return rc;
-        if (split_k > 64) split_k = 64;  // (the automatic choice may name a split the ordinary streams take)
+        // the automatic choice is the ordinary streams'; wide tiles do best with at most 32 lanes per column (K=13824 N=5120,
+        // 16 rows, 7 GEMVs per launch, split_k 32 / 64: u16 15.7 / 22.4 us per GEMV, gap stream 13.0 / 21.5)
+        if (pick && split_k > 32) split_k = 32;
         int bits = 0;
         size_t read_bytes = 0;
         uint64_t nnz = 0;
@@ -425,9 +475,12 @@ struct FileHeader {
     int32_t index_shift;      // u16 lists: fields are row << index_shift; 8-bit gap streams: 2 when the visiting order was scheduled for
                               // tiles of one byte per row (LDS bank = (row >> 2) mod 32), else 0
     uint64_t nnz, read_bytes, stream_bytes;
-    uint64_t fnv1a;           // of the header (this field zero) and the stream
+    uint64_t fnv1a;           // of the header (this field zero), the plans (version 3) and the stream
 };
 static_assert(sizeof(FileHeader) == 8 + 4 + 4 + 7 * 4 + 6 * 4 + 5 * 4 + 4 * 8, "file header has no padding");
+// version 3: the stream's launch plans follow the header (PLAN_SLOTS x 8 int32), then the stream
+typedef int32_t FilePlans[PLAN_SLOTS][8];
+static_assert(sizeof(FilePlans) == sizeof(Plan) * PLAN_SLOTS, "a plan is eight int32");
 const char FILE_MAGIC[8] = {'S', 'P', 'T', 'M', 'M', 'W', '1', 0};
 
 uint64_t fnv1a(const uint8_t *p, size_t n, uint64_t h = 1469598103934665603ull)
@@ -436,10 +489,12 @@ uint64_t fnv1a(const uint8_t *p, size_t n, uint64_t h = 1469598103934665603ull)
     return h;
 }
 
-uint64_t file_checksum(FileHeader h, const std::vector<uint8_t> &stream)
+uint64_t file_checksum(FileHeader h, const FilePlans *plans, const std::vector<uint8_t> &stream)
 {
     h.fnv1a = 0;
-    return fnv1a(stream.data(), stream.size(), fnv1a((const uint8_t *)&h, sizeof h));
+    uint64_t x = fnv1a((const uint8_t *)&h, sizeof h);
+    if (plans) x = fnv1a((const uint8_t *)plans, sizeof(FilePlans), x);
+    return fnv1a(stream.data(), stream.size(), x);
 }
 }  // namespace
 
@@ -452,7 +507,9 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
         FileHeader h{};
         memcpy(h.magic, FILE_MAGIC, 8);
         h.header_bytes = (uint32_t)sizeof h;
-        h.version = 2;
+        h.version = 3;
+        FilePlans plans;
+        memcpy(plans, w->plans, sizeof plans);
         const sptmm_winfo &i = w->info;
         const Geometry &g = w->geo;
         // ragged: 0 balanced, 1 ragged, 2 wide (K-tiled; the stream's own 512-byte header holds the tiles' offsets and counts)
@@ -461,10 +518,10 @@ int sptmm_weights_save(const sptmm_weights *w, const char *path)
         h.task_stride = w->task_stride, h.counts_bytes = w->counts_bytes, h.n_min = w->n_min, h.n_max = w->n_max;
         h.index_shift = i.kind == SPTMM_KIND_DELTA ? (w->byte_rows ? 2 : 0) : w->index_shift;
         h.nnz = i.nnz, h.read_bytes = i.stream_bytes, h.stream_bytes = w->bytes;
-        h.fnv1a = file_checksum(h, host);
+        h.fnv1a = file_checksum(h, &plans, host);
         FILE *f = fopen(path, "wb");
         if (!f) return fail(SPTMM_ERR_INVALID, "cannot open %s for writing", path);
-        const bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(host.data(), 1, host.size(), f) == host.size();
+        const bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(plans, sizeof plans, 1, f) == 1 && fwrite(host.data(), 1, host.size(), f) == host.size();
         if (fclose(f) != 0 || !ok) return fail(SPTMM_ERR_INVALID, "short write to %s", path);
         return SPTMM_OK;
     });
@@ -479,7 +536,9 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         FileHeader h{};
         std::vector<uint8_t> host;
         int rc = SPTMM_OK;
-        if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || (h.version != 1 && h.version != 2))
+        FilePlans plans = {};
+        if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, FILE_MAGIC, 8) != 0 || h.header_bytes != sizeof h || h.version < 1 || h.version > 3 ||
+            (h.version == 3 && fread(plans, sizeof plans, 1, f) != 1))
             rc = fail(SPTMM_ERR_INVALID, "%s is not a weight file of this library", path);
         // every field the kernels index with is checked against the stream size before anything is uploaded
         if (!rc) {
@@ -526,7 +585,7 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
             host.resize(h.stream_bytes);
             if (fread(host.data(), 1, host.size(), f) != host.size() || fgetc(f) != EOF)
                 rc = fail(SPTMM_ERR_INVALID, "%s: truncated or oversized file", path);
-            else if (file_checksum(h, host) != h.fnv1a)
+            else if (file_checksum(h, h.version == 3 ? &plans : nullptr, host) != h.fnv1a)
                 rc = fail(SPTMM_ERR_INVALID, "%s: checksum mismatch", path);
         }
         fclose(f);
@@ -576,6 +635,7 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         if (!w) return fail(SPTMM_ERR_NOMEM, "out of host memory");
         w->info = sptmm_winfo{h.kind, h.K, h.N, h.S, h.split_k, h.delta_bits, h.read_bytes, h.ragged ? 1 : 0, h.nnz};
         w->geo = Geometry{h.N, h.half, h.split_k, h.L, h.G, h.W, h.n_lane, h.tasks};
+        memcpy(w->plans, plans, sizeof plans);  // (values a kernel cannot take are ignored at launch)
         if (h.ragged == 2) {
             w->wide = true;
             w->wh = wh;
@@ -592,6 +652,123 @@ int sptmm_weights_load(const char *path, sptmm_weights **out)
         w->stones = h.ragged && h.kind == SPTMM_KIND_DELTA && h.delta_bits == 8 && *(const uint32_t *)host.data() == RAGGED_MAGIC_STONES;
         w->info.stones = w->stones ? 1 : 0;
         return finish_upload(w, host, out);
+    });
+}
+
+int sptmm_weights_set_plan(sptmm_weights *w, int M, int batched, const sptmm_plan *plan)
+{
+    if (!w || !plan) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    memcpy(&w->plans[plan_slot(M, batched != 0)], plan, sizeof(Plan));
+    return SPTMM_OK;
+}
+
+int sptmm_weights_get_plan(const sptmm_weights *w, int M, int batched, sptmm_plan *out)
+{
+    if (!w || !out) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    memcpy(out, &w->plans[plan_slot(M, batched != 0)], sizeof(Plan));
+    return SPTMM_OK;
+}
+
+int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_model, double *us_tuned)
+{
+    return guarded([&]() -> int {
+        if (!w) return fail(SPTMM_ERR_INVALID, "null pointer");
+        if (M < 1 || batch < 0) return fail(SPTMM_ERR_INVALID, "M must be at least 1 and batch at least 0");
+        if (act < ACT_I8 || act > ACT_F32) return fail(SPTMM_ERR_INVALID, "act must be 0 (int8), 1 (fp16) or 2 (fp32)");
+        if (w->info.kind == SPTMM_KIND_I2S && act != ACT_I8) return fail(SPTMM_ERR_UNSUPPORTED, "the i2s kernel takes int8 activations only");
+        const bool batched = batch > 0, lists = w->info.kind != SPTMM_KIND_I2S && !w->wide;
+        const int slot = plan_slot(M, batched);
+        // device copies to rotate over: the batch itself, or enough for ~300 MB
+        const int n = batched ? std::min(batch, 32) : (int)std::max<size_t>(2, std::min<size_t>(32, (300u << 20) / std::max<size_t>(w->bytes, 1) + 1));
+        std::vector<sptmm_weights *> owned;
+        std::vector<const sptmm_weights *> ws{w};
+        void *X = nullptr, *C = nullptr, *stream = nullptr;
+        int rc = SPTMM_OK;
+        auto cleanup = [&] {
+            for (sptmm_weights *c : owned) sptmm_weights_free(c);
+            if (X) (void)hipFree(X);
+            if (C) (void)hipFree(C);
+            if (stream) (void)hipStreamDestroy((hipStream_t)stream);
+        };
+        for (int i = 1; i < n && rc == SPTMM_OK; ++i) {
+            sptmm_weights *c = nullptr;
+            rc = sptmm_weights_clone(w, &c);
+            if (rc == SPTMM_OK) owned.push_back(c), ws.push_back(c);
+        }
+        const size_t xbytes = (size_t)M * w->info.K * (act == ACT_I8 ? 1 : act == ACT_F16 ? 2 : 4), cbytes = (size_t)4 * M * w->info.N * (batched ? n : 1);
+        if (rc == SPTMM_OK) rc = sptmm_malloc(&X, xbytes);
+        if (rc == SPTMM_OK) rc = sptmm_malloc(&C, cbytes);
+        if (rc == SPTMM_OK) rc = sptmm_memset(X, 0, xbytes);
+        if (rc == SPTMM_OK) rc = sptmm_stream_create(&stream);
+        if (rc != SPTMM_OK) {
+            cleanup();
+            return rc;
+        }
+        // microseconds per GEMV under `plan`: best of three short loops after a rotation of warm-up
+        auto time_plan = [&](const Plan &plan, double *us) -> int {
+            w->plans[slot] = plan;
+            for (sptmm_weights *c : owned) c->plans[slot] = plan;
+            const int iters = batched ? 6 * n : std::max(3 * n, 48);
+            double best = 1e30, t = 0;
+            if (int r = measure_gemv(ws.data(), n, act, X, M, C, batched ? n : n, batched ? 3 : 0, stream, &t)) return r;
+            for (int rep = 0; rep < 3; ++rep) {
+                if (int r = measure_gemv(ws.data(), n, act, X, M, C, iters, batched ? 3 : 0, stream, &t)) return r;
+                best = std::min(best, t);
+            }
+            *us = best;
+            return SPTMM_OK;
+        };
+        const Plan before = w->plans[slot];
+        Plan best{};
+        double t_model = 0, t_best = 0;
+        rc = time_plan(best, &t_model);
+        t_best = t_model;
+        // one dimension at a time, each from the best plan so far
+        struct Dim {
+            int Plan::*field;
+            std::vector<int> values;
+        };
+        std::vector<Dim> dims;
+        if (w->info.kind == SPTMM_KIND_I2S) {
+            dims.push_back({&Plan::i2s_ct, {1, 2, 4, 8}});
+            dims.push_back({&Plan::waves_per_wg, {1, 2, 4, 8}});
+        } else if (w->wide) {
+            dims.push_back({&Plan::waves_per_wg, {4, 6, 8, 10, 12, 16}});
+        } else if (batched) {
+            dims.push_back({&Plan::waves_per_wg, {2, 4, 5, 6, 8, 10, 12, 16}});
+            dims.push_back({&Plan::tasks_per_wave, {1, 2, 3, 4, 5, 6, 8, 10, 12, 16}});
+        } else {
+            dims.push_back({&Plan::waves_per_wg, {2, 4, 5, 6, 8, 10, 12, 16}});
+            dims.push_back({&Plan::wgs_per_cu, {1, 2, 3}});
+            if (lists && w->info.kind == SPTMM_KIND_U16 && M == 1 && act == ACT_I8) dims.push_back({&Plan::share_log, {-1, 1, 2}});
+        }
+        for (const Dim &d : dims)
+            for (int v : d.values) {
+                if (rc != SPTMM_OK) break;
+                Plan p = best;
+                p.*(d.field) = v;
+                double t = 0;
+                rc = time_plan(p, &t);
+                if (rc == SPTMM_OK && t < t_best) t_best = t, best = p;
+            }
+        if (rc == SPTMM_OK) {
+            // the model's shape stays unless the search found something at least 2 % faster, confirmed by a second timing
+            if (t_best < 0.98 * t_model) {
+                double again = 0;
+                rc = time_plan(best, &again);
+                if (rc == SPTMM_OK && again >= 0.98 * t_model) best = Plan{}, t_best = t_model;
+                else if (rc == SPTMM_OK) t_best = std::min(t_best, again);
+            } else {
+                best = Plan{}, t_best = t_model;
+            }
+        }
+        w->plans[slot] = rc == SPTMM_OK ? best : before;
+        if (us_model) *us_model = t_model;
+        if (us_tuned) *us_tuned = t_best;
+        cleanup();
+        return rc;
     });
 }
 

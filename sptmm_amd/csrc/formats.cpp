@@ -26,13 +26,11 @@ void tuning_reload()
         return v && *v ? atoi(v) : otherwise;
     };
     Tuning t;
-    t.waves_per_wg = knob("SPTMM_WAVES_PER_WG", 0);
-    t.wgs_per_cu = knob("SPTMM_WGS_PER_CU", 0);
-    t.tasks_per_wave = knob("SPTMM_TASKS_PER_WAVE", 0);
-    t.share_log = knob("SPTMM_SHARE_LOG", 0);
-    t.wide_waves = knob("SPTMM_WIDE_WAVES", 0);
-    t.i2s_waves = knob("SPTMM_I2S_WAVES", 0);
-    t.i2s_ct = knob("SPTMM_I2S_CT", 0);
+    t.plan.waves_per_wg = knob("SPTMM_WAVES_PER_WG", 0);
+    t.plan.wgs_per_cu = knob("SPTMM_WGS_PER_CU", 0);
+    t.plan.tasks_per_wave = knob("SPTMM_TASKS_PER_WAVE", 0);
+    t.plan.share_log = knob("SPTMM_SHARE_LOG", 0);
+    t.plan.i2s_ct = knob("SPTMM_I2S_CT", 0);
     t.i2s_mfma_from = knob("SPTMM_I2S_MFMA_FROM", 2);
     g_tuning = t;
 }

@@ -400,7 +400,7 @@ static int launch_i2s_mfma_t(const GemvArgs &a, hipStream_t st, int waves)
 
 static int launch_i2s_mfma(const GemvArgs &a, hipStream_t st)
 {
-    const int tune_waves = tuning().i2s_waves, tune_ct = tuning().i2s_ct;
+    const int tune_waves = a.plan.waves_per_wg, tune_ct = a.plan.i2s_ct;
     const int rounds = i2s_padded_k(a.K) / 256, groups = a.N / 16;
     const int rows = a.M < 16 ? a.M : 16, xj = (rows + 3) / 4;  // loads of X rows per round: four rows each
     // Column tiles per wavefront and wavefronts per workgroup, measured on MI355X (K=6912 N=2560 and K=13824

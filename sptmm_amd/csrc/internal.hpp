@@ -151,6 +151,30 @@ inline int i2s_padded_k(int K) { return (K + 255) / 256 * 256; }
 // ---- validation shared by packers and uploaders -----------------------------
 int check_shape(int K, int N, int S);
 
+// The launch shape of one kind of call on one stream, where it is not left to the launchers' own model: every field 0 =
+// the model's choice.  Mirrors sptmm_plan (sptmm.h) field for field.
+struct Plan {
+    int waves_per_wg = 0;    // wavefronts per workgroup (list and wide kernels; i2s: of the matrix-unit kernel)
+    int wgs_per_cu = 0;      // workgroups per compute unit of a lone list launch
+    int tasks_per_wave = 0;  // tasks per wavefront of a batched list launch
+    int share_log = 0;       // a lone GEMV (one int8 row, u16 lists): 1 << this many wavefronts per task; -1: never
+    int i2s_ct = 0;          // column tiles per wavefront of the i2s matrix-unit kernel
+    int reserved[3] = {0, 0, 0};
+};
+static_assert(sizeof(Plan) == sizeof(sptmm_plan), "Plan mirrors sptmm_plan");
+// Which of a stream's plans a call takes: by its activation rows (1, 2-4, 5-8, more) and by whether it is a batched launch.
+constexpr int PLAN_SLOTS = 8;
+inline int plan_slot(int M, bool batched) { return 2 * (M <= 1 ? 0 : M <= 4 ? 1 : M <= 8 ? 2 : 3) + (batched ? 1 : 0); }
+
+// Process-wide launch-shape overrides for tuning runs, under a stream's own plan.  Filled from the environment by
+// sptmm_device_init -- once per call of it, never on a launch path -- and by nothing else.
+struct Tuning {
+    Plan plan;               // SPTMM_WAVES_PER_WG, SPTMM_WGS_PER_CU, SPTMM_TASKS_PER_WAVE, SPTMM_SHARE_LOG, SPTMM_I2S_CT
+    int i2s_mfma_from = 2;   // SPTMM_I2S_MFMA_FROM: rows from which a lone i2s launch takes the matrix-unit kernel
+};
+const Tuning &tuning();
+void tuning_reload();  // reads the environment (formats.cpp)
+
 // ---- device-side launchers (i2s.hip and the lists_*.hip files) --------------------------------------
 struct GemvArgs {
     const void *w;      // device stream
@@ -175,23 +199,9 @@ struct GemvArgs {
     size_t batch_w_skip = 0;  // bytes in front of every batch_w[i] that the kernels do not read (a count table they need not look at)
     const void *const *batch_X = nullptr;
     void *const *batch_C = nullptr;
+    Plan plan;            // launch-shape overrides: the stream's plan for this kind of call over the process-wide ones
 };
 enum ActType { ACT_I8 = 0, ACT_F16 = 1, ACT_F32 = 2 };
-
-// Launch-shape overrides for tuning runs (0 = the launcher's own choice).  Filled from the environment by
-// sptmm_device_init -- once per call of it, never on a launch path -- and by nothing else.
-struct Tuning {
-    int waves_per_wg = 0;    // SPTMM_WAVES_PER_WG: wavefronts per workgroup of the list kernels
-    int wgs_per_cu = 0;      // SPTMM_WGS_PER_CU: workgroups per compute unit of a lone list launch
-    int tasks_per_wave = 0;  // SPTMM_TASKS_PER_WAVE: tasks per wavefront of a batched list launch
-    int wide_waves = 0;      // SPTMM_WIDE_WAVES: wavefronts per workgroup of the wide kernels
-    int i2s_waves = 0;       // SPTMM_I2S_WAVES
-    int i2s_ct = 0;          // SPTMM_I2S_CT: column tiles per wavefront of the i2s matrix-unit kernel
-    int i2s_mfma_from = 2;   // SPTMM_I2S_MFMA_FROM: rows from which a lone i2s launch takes the matrix-unit kernel
-    int share_log = 0;       // SPTMM_SHARE_LOG: a lone GEMV (one int8 row, u16 lists) gives each task 1 << this many wavefronts
-};
-const Tuning &tuning();
-void tuning_reload();  // reads the environment (formats.cpp)
 
 int launch_u16(const GemvArgs &a, ActType act, void *stream);
 int launch_u16_scaled(const GemvArgs &a, ActType act, void *stream);   // lists_u16_scaled.hip

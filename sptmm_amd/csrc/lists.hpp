@@ -1219,8 +1219,8 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // tiles take.  Measured on MI355X, K=2560 N=13824 split_k=32: one workgroup per CU 11.4 us,
     // two 6.3 us; the headline shape has 5 tasks per CU and stays at one workgroup of 5.
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
-    // launch-shape overrides for tuning runs (the environment as sptmm_device_init last read it)
-    const int tune_wpb = tuning().waves_per_wg, tune_wgs = tuning().wgs_per_cu, tune_tpw = tuning().tasks_per_wave;
+    // launch-shape overrides: the stream's plan for this kind of call, else what sptmm_device_init read from the environment
+    const int tune_wpb = a.plan.waves_per_wg, tune_wgs = a.plan.wgs_per_cu, tune_tpw = a.plan.tasks_per_wave;
     constexpr int SLOT = slot_bytes<Act, MT>();
     const size_t tile = (size_t)(lists_tile_rows(a) + 64) * SLOT;
     // batched launches fill the CU with several workgroups where two tiles fit; then the smaller ones do better
@@ -1250,7 +1250,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             const int iters = (blocks + grid - 1) / grid;
             const double r = (double)g * w;
             // + each workgroup stages the tile once; a bubble per extra pass; when latency-bound, spread over more CUs
-            const double cost = iters * (r > r_lat ? r : r_lat) + 0.05 * g + 0.25 * (iters - 1) + 0.001 * r;
+            // (where the latency term leaves several workgroup sizes level, four or five wavefronts: a lone launch of few
+            // tasks does better in a few such workgroups than in one or two wavefronts on every compute unit -- K=4352
+            // N=512 S=992, 128 tasks: 3.64 -> 3.20 us in workgroups of five; K=6400 N=2048 S=1952, gap stream: 4.39 -> 3.94)
+            const double cost = iters * (r > r_lat ? r : r_lat) + 0.05 * g + 0.25 * (iters - 1) + 0.001 * (w < 4 ? 4.5 - w : w - 4.5);
             if (cost < best - 1e-9) {
                 best = cost;
                 wpb = w;
@@ -1266,6 +1269,18 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // u16 lists on one- and four-row int8 tiles, batched, more tasks than the headline shape's 1280: eight wavefronts
     // (K=13824 N=5120: M=1 12.9 -> 12.3 us per GEMV, M=4 13.5 -> 12.6; K=2560 N=6912, M=4: 3.2 -> 3.0 us)
     if (MODE == 0 && MT <= 4 && sizeof(Act) == 1 && !is_byte_rows<Act>() && a.batch >= 4 && a.W == 1 && a.tasks >= 1536 && max_waves >= 8) wpb = 8;
+    // ... and for the other shapes of those launches: what streams is the number of wavefronts a compute unit holds, and the
+    // tile decides how many workgroups fit one.  At least 24 wavefronts per compute unit, in workgroups of at least four
+    // (the latency model above counts tasks in flight and would take two or three wavefronts per 46 KB tile).  16 GEMVs per
+    // launch, model's pick -> this: K=11520 N=2816 S=1536 M=1 1.67 -> 1.39 us per GEMV, M=4 2.04 -> 1.43; K=6400 N=2048
+    // S=1952 1.54 -> 1.29, M=4 1.77 -> 1.35; K=4352 N=512 S=992 0.38 -> 0.29; K=4096 N=4352 S=1856 2.76 -> 2.44.
+    else if (MODE == 0 && MT <= 4 && sizeof(Act) == 1 && !is_byte_rows<Act>() && a.batch >= 4 && a.W == 1 && max_waves >= 8) {
+        // Four or eight, which the four SIMDs share evenly: four where six or more tiles fit a compute unit, eight where
+        // four or fewer do (K=4096 N=4352 S=1856, 5 -> 4 wavefronts: 2.76 -> 2.38 us; K=8704 N=3328 S=1408, 6 -> 8: 1.93 -> 1.68).
+        const int by_lds = std::max(1, (int)((size_t)a.lds_limit / (tile + lists_behind_tile<Act, MT>(LISTS_MAX_WAVES))));
+        if (by_lds >= 6) wpb = 4;
+        else if (by_lds <= 4) wpb = 8;
+    }
     // eight-row tiles keep the matrix unit busy: a batched launch takes a wavefront count the four SIMDs share evenly
     // (K=13824 N=5120, M=8, 10 -> 12 wavefronts: gap stream 48 -> 55 % of HBM peak, u16 lists level)
     // -- and the largest workgroup does best: four wavefronts per SIMD, fewer workgroups staging (same shape, 12 -> 16
@@ -1279,6 +1294,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // for fp16 rows (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824
     // five do better)
     if (MT == 4 && MODE != 0 && a.batch >= 4 && a.W == 1 && tile <= 40 * 1024 && max_waves >= 8) wpb = sizeof(Act) == 1 ? 4 : 8;
+    // ... four int8 rows on tiles of more than 30 KB: two workgroups or fewer per compute unit would leave it eight
+    // wavefronts; the largest workgroup instead (16 GEMVs per launch: K=11520 N=2816 S=1536 1.85 -> 1.05 us per GEMV,
+    // K=8704 N=3328 S=1408 1.75 -> 1.13)
+    if (MT == 4 && MODE != 0 && sizeof(Act) == 1 && a.batch >= 4 && a.W == 1 && tile > 30 * 1024) wpb = lists_max_waves<Act, MT, false>();
     // four fp16 rows (sums on the matrix unit, 56 KB tile at K=6912), batched: eight wavefronts as well
     // (headline shape, 5 -> 8: u16 lists 69 -> 81 % of HBM peak, gap stream 39 -> 53 %)
     if (MT == 4 && sizeof(Act) == 2 && a.batch >= 4 && a.W == 1 && max_waves >= 8) wpb = 8;
@@ -1312,7 +1331,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         const int resident = std::max(1, std::min(by_lds, by_regs));
         const long at_once = (long)cus * resident;
         const int row_tiles = (a.M + MT - 1) / MT;
-        const double stage = WIDE_SLOT ? 2.5 : 2.0, walk = WIDE_SLOT ? 4.0 : 5.7;
+        // (the two costs as measured on a 110 KB tile with 8.6 KB tasks, and on a 28 KB tile with 8.4 KB tasks; other
+        // shapes in proportion to their tile and task bytes)
+        const double stage = (WIDE_SLOT ? 2.5 / 110.0 : 2.0 / 28.0) * ((double)tile / 1024.0);
+        const double walk = (WIDE_SLOT ? 4.0 / 8.6 : 5.7 / 8.4) * task_kb;
         double best = 1e30;
         int pick = iters;
         for (int t = 1; t <= 16 && t <= blocks; ++t) {
@@ -1327,7 +1349,8 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         }
         grid_x = (blocks + pick - 1) / pick;
         iters = (blocks + grid_x - 1) / grid_x;
-    } else if (a.batch >= 8 && iters == 1 && blocks >= 2 && !(MODE == 0 && (MT == 1 || (MT == 4 && sizeof(Act) == 1))) &&
+    } else if (a.batch >= 8 && iters == 1 && blocks >= 2 && (long)a.batch * ((blocks + 1) / 2) >= 2L * cus &&  // (still two workgroups per compute unit)
+               !(MODE == 0 && (MT == 1 || (MT == 4 && sizeof(Act) == 1))) &&
                !(is_byte_rows<Act>() && !VAR && task_kb >= 8.0 && tile <= (size_t)(task_kb * 1024.0))) {
         // (byte rows whose task is 8 KB or more and no smaller than the tile: one task per wavefront, 1.54 against 1.63 us
         // on the headline shape; shorter tasks and larger tiles do better with two)
@@ -1417,7 +1440,7 @@ static bool try_shared(const GemvArgs &a, hipStream_t st, int *rc)
     if constexpr (std::is_same<Act, int8_t>::value && MT == 1 && MODE == 0 && !VAR) {
         if (a.batch || a.quant || a.W != 1 || a.M != 1) return false;
         const int rounds = a.n_lane / 8, cus = a.compute_units > 0 ? a.compute_units : 256;
-        int sl = tuning().share_log, wpb = tuning().waves_per_wg;
+        int sl = a.plan.share_log, wpb = a.plan.waves_per_wg;
         if (sl < 0 || rounds < 2 || rounds > 8) return false;
         if (sl == 0) {
             // two wavefronts per task where the doubled launch is at most ten wavefronts per compute unit, in workgroups that

@@ -268,13 +268,14 @@ template <typename Act, int MODE, int RING_ = 4> struct WideBody {
     // keeps its wavefront), by the same lane as long as the phases sum on the same unit; where an fp16 tile holds a
     // non-finite value and the phase sums on the vector unit, another lane of that wavefront writes it.  Either way the
     // earlier store is complete and in L2 before the later load: every phase but the first starts with a workgroup
-    // barrier, which waits for the wavefront's outstanding stores, and both the store and the load are agent-scope
-    // atomics (relaxed), which go to L2 rather than stay in the compute unit's own cache.
+    // barrier, which waits for the wavefront's outstanding stores (the compute unit's own cache writes through), and
+    // the load is an agent-scope atomic, served by L2.  (An agent-scope atomic store as well costs 5-7 % of a batched
+    // 16-row launch at K=13824 and adds nothing to that.)
     static __device__ __forceinline__ void put(const WideParams &p, void *C, int m, int col, A v, bool first)
     {
         A *c = reinterpret_cast<A *>(C) + (size_t)m * p.N + col;
         if (!first) v += __hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(c, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *c = v;
     }
 
     // (w, Xv, C: the launch's stream, activations and output; a batched launch picks them per blockIdx.z and leaves
@@ -381,7 +382,7 @@ template <typename Act, int MODE, int RING, int MAXW>
 static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
 {
     constexpr int ROWS = WideSums<Act>::ROWS;
-    const int tune_wpb = tuning().wide_waves;
+    const int tune_wpb = a.plan.waves_per_wg;
     const int cus = a.compute_units > 0 ? a.compute_units : 256;
     const size_t lds = (size_t)(h.k_tile + 64) * 16 + 64;
     if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "the stream's K-tile of %d rows needs %zu bytes of LDS, the device grants %d", h.k_tile, lds, a.lds_limit);

@@ -27,7 +27,7 @@ def test_final_line_of_a_full_run_is_short_and_keeps_the_contract():
     import bench
 
     full = json.load(open(os.path.join(ROOT, "tests", "golden", "bench_full_sample.json")))
-    for leg in ("single_launch", "other_encodings", "configs", "density_sweep", "cpu_baseline", "layer_sequence"):
+    for leg in ("single_launch", "other_encodings", "configs", "density_sweep", "cpu_baseline", "layer_sequence", "launch_plans"):
         assert full.get(leg), leg
     assert len(json.dumps(full)) > 4 * LINE_LIMIT  # the sample really holds the tables
     line = bench.final_line(full)
@@ -40,7 +40,7 @@ def test_final_line_of_a_full_run_is_short_and_keeps_the_contract():
     for k in ("value", "unit", "cores", "kind", "sample"):
         assert k in j["cpu_baseline"], k
     assert "configs" not in j and "density_sweep" not in j
-    for k in ("cfg1_m4", "cfg2_delta_fp16", "cfg3_layer_summed", "cfg4_large", "layer_sequence", "density_lists_over_i2s"):
+    for k in ("cfg1_m4", "cfg2_delta_fp16", "cfg3_layer_summed", "cfg4_large", "layer_sequence", "density_lists_over_i2s", "launch_plans_model_vs_tuned"):
         assert k in j["summary"], k
 
 
@@ -57,7 +57,7 @@ def test_json_line_has_the_contract_keys(tmp_path):
     for k in CONTRACT_KEYS:
         assert k in j, k
     full = json.load(open(detail))
-    assert full["configs"]["cfg3_layer"]["shapes"] and full["density_sweep"]["shapes"] and full["layer_sequence"]["rows"]
+    assert full["configs"]["cfg3_layer"]["shapes"] and full["density_sweep"]["shapes"] and full["layer_sequence"]["rows"] and full["launch_plans"]["rows"]
     assert "layer_sequence" in j["summary"] and "cfg4_large" in j["summary"]
     assert j["n_gpus"] == 1 and j["steps"] == 8 and j["warmup"] == 2 and j["higher_is_better"] is False and j["vs_baseline"] is None
     assert "workload" in j["config"] and "model" not in j["config"]

@@ -162,6 +162,33 @@ def test_non_finite_value_in_one_k_tile_only(bad):
         w.free()
 
 
+def test_uploads_that_declare_more_than_eight_rows_build_wide_streams():
+    """The _rows upload calls build the stream for the rows a call will bring: beyond eight, a wide stream (the lists read
+    once for up to 16 rows); up to eight, the ordinary one.  Whichever it is, the sums are the oracle's at any M."""
+    K, N, S = 2560, 640, 1536
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    made = {
+        "u16 rows=16": sp.Weights.upload_u16(pos, neg, K, 0, rows=16),
+        "u16 rows=9, split 32": sp.Weights.upload_u16(pos, neg, K, 32, rows=9),
+        "delta rows=16": sp.Weights.upload_delta(pos, neg, K, 0, rows=16),
+        "dense u16 rows=12": sp.Weights.upload_dense(W, sp.KIND_U16, 0, rows=12),
+        "dense delta rows=16": sp.Weights.upload_dense(W, sp.KIND_DELTA, 16, rows=16),
+        "u16 rows=8": sp.Weights.upload_u16(pos, neg, K, 0, rows=8),
+        "delta rows=8": sp.Weights.upload_delta(pos, neg, K, 0, rows=8),
+        "u16 rows=16, split 128": sp.Weights.upload_u16(pos, neg, K, 128, rows=16),  # wide streams stop at 64 lanes per column
+    }
+    for name, w in made.items():
+        wide = "rows=8" not in name and "split 128" not in name
+        say("declared rows:", name, "k_tile", w.info["k_tile"])
+        assert (w.info["k_tile"] != 0) == wide, name
+        if wide and "dense" not in name:
+            assert w.info["S"] == S
+        for M in (1, 9, 16):
+            X = oracle.make_x_i8(M, M, K)
+            assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), (name, M)
+        w.free()
+
+
 def test_refusals():
     K, N = 512, 48
     W = sp.generate_ternary_iid(K, N, 1, 0.3, 0.3)

@@ -8,6 +8,10 @@ import pytest
 import oracle
 import sptmm_amd as sp
 
+HEADER = 120          # the fixed header
+PLANS = 8 * 8 * 4     # version 3: the stream's launch plans (8 kinds of call x 8 int32) between header and stream
+DATA = HEADER + PLANS
+
 
 def test_load_refuses_what_is_not_a_weight_file(tmp_path):
     # these are rejected from the header alone, before any device call
@@ -53,7 +57,7 @@ def test_save_load_round_trip_every_encoding(tmp_path):
         want = w.matmul(X)
         path = str(tmp_path / (name + ".sptmm"))
         w.save(path)
-        assert os.path.getsize(path) == 120 + w.nbytes
+        assert os.path.getsize(path) == DATA + w.nbytes
         v = sp.Weights.load(path)
         assert v.info == w.info and v.nbytes == w.nbytes
         assert (v.matmul(X) == want).all()
@@ -62,12 +66,18 @@ def test_save_load_round_trip_every_encoding(tmp_path):
         v.free()
         # one flipped stream byte, a truncated file and trailing bytes are all refused
         raw = bytearray(open(path, "rb").read())
-        raw[120 + len(raw) // 3] ^= 0x40
+        raw[DATA + len(raw) // 3] ^= 0x40
         open(path, "wb").write(bytes(raw))
         with pytest.raises(sp.SptmmError) as e:
             sp.Weights.load(path)
         assert "checksum" in str(e.value) or "corrupt" in str(e.value)
-        raw[120 + len(raw) // 3] ^= 0x40
+        raw[DATA + len(raw) // 3] ^= 0x40
+        raw[HEADER + 5] ^= 1  # ... and so is a flipped byte of the plans
+        open(path, "wb").write(bytes(raw))
+        with pytest.raises(sp.SptmmError) as e:
+            sp.Weights.load(path)
+        assert "checksum" in str(e.value)
+        raw[HEADER + 5] ^= 1
         open(path, "wb").write(bytes(raw[:-5]))
         with pytest.raises(sp.SptmmError):
             sp.Weights.load(path)
@@ -103,17 +113,26 @@ def test_version_1_i2s_file_is_retiled_on_load(tmp_path):
     w.save(path)
     w.free()
     raw = bytearray(open(path, "rb").read())
-    assert int.from_bytes(raw[12:16], "little") == 2
-    stream = np.frombuffer(bytes(raw[120:]), np.uint8).reshape(-1, 4, 16, 16)      # [tile][q][c][16 bytes]
+    assert int.from_bytes(raw[12:16], "little") == 3
+    stream = np.frombuffer(bytes(raw[DATA:]), np.uint8).reshape(-1, 4, 16, 16)     # [tile][q][c][16 bytes]
     old = np.ascontiguousarray(stream.transpose(0, 2, 1, 3)).tobytes()             # [tile][c][q][16 bytes]
     hdr = bytearray(raw[:120])
     hdr[12:16] = (1).to_bytes(4, "little")
     hdr[112:120] = bytes(8)
     hdr[112:120] = _fnv1a(bytes(hdr) + old).to_bytes(8, "little")
     p1 = str(tmp_path / "v1.sptmm")
-    open(p1, "wb").write(bytes(hdr) + old)
+    open(p1, "wb").write(bytes(hdr) + old)  # versions 1 and 2 have no plans behind the header
     v = sp.Weights.load(p1)
     assert (v.matmul(X) == oracle.dense_i8(X, W)).all()
+    v.free()
+    # version 2: the current tile order, still without plans
+    hdr[12:16] = (2).to_bytes(4, "little")
+    hdr[112:120] = bytes(8)
+    hdr[112:120] = _fnv1a(bytes(hdr) + bytes(raw[DATA:])).to_bytes(8, "little")
+    p2 = str(tmp_path / "v2.sptmm")
+    open(p2, "wb").write(bytes(hdr) + bytes(raw[DATA:]))
+    v = sp.Weights.load(p2)
+    assert (v.matmul(X) == oracle.dense_i8(X, W)).all() and not any(v.get_plan(1, False).values())
     v.free()
 
 
@@ -133,19 +152,19 @@ def test_wide_file_with_a_bad_table_is_refused_although_its_checksum_holds(tmp_p
     v.free()
     w.free()
     raw = bytearray(open(path, "rb").read())
-    hdr = np.frombuffer(bytes(raw[120:120 + 512]), np.uint32)
+    hdr = np.frombuffer(bytes(raw[DATA:DATA + 512]), np.uint32)
     off = int(hdr[8])
     damages = {
-        "count above n_max": (120 + off + 16, (65535).to_bytes(2, "little")),
-        "offset past the stream": (120 + 4 * 8, (len(raw)).to_bytes(4, "little")),
-        "stride": (120 + 4 * 9, (int(hdr[9]) + 128).to_bytes(4, "little")),
-        "k_tile": (120 + 4 * 2, (16320).to_bytes(4, "little")),
-        "phases": (120 + 4 * 1, (3).to_bytes(4, "little")),
+        "count above n_max": (DATA + off + 16, (65535).to_bytes(2, "little")),
+        "offset past the stream": (DATA + 4 * 8, (len(raw)).to_bytes(4, "little")),
+        "stride": (DATA + 4 * 9, (int(hdr[9]) + 128).to_bytes(4, "little")),
+        "k_tile": (DATA + 4 * 2, (16320).to_bytes(4, "little")),
+        "phases": (DATA + 4 * 1, (3).to_bytes(4, "little")),
     }
     for what, (at, val) in damages.items():
         bad = bytearray(raw)
         bad[at:at + len(val)] = val
-        bad[112:120] = bytes(8)                      # the checksum covers the header with this field zero, then the stream
+        bad[112:120] = bytes(8)                      # the checksum covers the header with this field zero, the plans, then the stream
         bad[112:120] = _fnv1a(bytes(bad)).to_bytes(8, "little")
         open(path, "wb").write(bytes(bad))
         with pytest.raises(sp.SptmmError) as e:
