@@ -232,7 +232,7 @@ size_t sptmm_weights_bytes(const sptmm_weights *w);
  * 0 = the model's choice; a value the kernels cannot take is ignored, never an error, and no plan changes a result.
  * The reference fixes its launch shapes at compile time (grid and block per instantiation, main.cu:996-1455).
  *   sptmm_weights_tune: a bounded search on the device -- a few dozen candidate plans, each timed over launches that
- *   rotate over device copies of the stream (HBM-cold; `batch` = 0 times lone launches, else launches of `batch`
+ *   rotate over enough device copies of the stream to exceed the last-level cache (`batch` = 0 times lone launches, else launches of `batch`
  *   GEMVs; act as in sptmm_gemv_batched; int8, fp16 or fp32 rows of zeros) -- which stores the fastest as the stream's
  *   plan for that kind of call and reports microseconds per GEMV under the model's shape and under the plan kept (the
  *   model's shape is kept unless a candidate is at least 2 % faster).  Synchronous; allocates and frees its own buffers.

@@ -32,9 +32,6 @@ struct sptmm_weights {
 
 namespace {
 
-int measure_gemv(const sptmm_weights *const *ws, int n_ws, int act, const void *X, int M, void *C, int iters, int mode, void *stream,
-                 double *us_per_call);
-
 int hip_fail(hipError_t e, const char *what)
 {
     return fail(SPTMM_ERR_HIP, "%s: %s (%d)", what, hipGetErrorString(e), (int)e);
@@ -680,16 +677,22 @@ int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_m
         if (w->info.kind == SPTMM_KIND_I2S && act != ACT_I8) return fail(SPTMM_ERR_UNSUPPORTED, "the i2s kernel takes int8 activations only");
         const bool batched = batch > 0, lists = w->info.kind != SPTMM_KIND_I2S && !w->wide;
         const int slot = plan_slot(M, batched);
-        // device copies to rotate over: the batch itself, or enough for ~300 MB
-        const int n = batched ? std::min(batch, 32) : (int)std::max<size_t>(2, std::min<size_t>(32, (300u << 20) / std::max<size_t>(w->bytes, 1) + 1));
+        // device copies to rotate over: enough for ~300 MB (more than the last-level cache holds), in whole batches
+        const int per = batched ? std::min(batch, 32) : 1;
+        const int by_bytes = (int)std::min<size_t>(64, (300u << 20) / std::max<size_t>(w->bytes, 1) + 1);
+        const int groups = std::max(batched ? 1 : 2, (by_bytes + per - 1) / per);
+        const int n = groups * per;
         std::vector<sptmm_weights *> owned;
         std::vector<const sptmm_weights *> ws{w};
         void *X = nullptr, *C = nullptr, *stream = nullptr;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
         int rc = SPTMM_OK;
         auto cleanup = [&] {
             for (sptmm_weights *c : owned) sptmm_weights_free(c);
             if (X) (void)hipFree(X);
             if (C) (void)hipFree(C);
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
             if (stream) (void)hipStreamDestroy((hipStream_t)stream);
         };
         for (int i = 1; i < n && rc == SPTMM_OK; ++i) {
@@ -697,25 +700,44 @@ int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_m
             rc = sptmm_weights_clone(w, &c);
             if (rc == SPTMM_OK) owned.push_back(c), ws.push_back(c);
         }
-        const size_t xbytes = (size_t)M * w->info.K * (act == ACT_I8 ? 1 : act == ACT_F16 ? 2 : 4), cbytes = (size_t)4 * M * w->info.N * (batched ? n : 1);
+        const size_t xbytes = (size_t)M * w->info.K * (act == ACT_I8 ? 1 : act == ACT_F16 ? 2 : 4), cbytes = (size_t)4 * M * w->info.N * per;
         if (rc == SPTMM_OK) rc = sptmm_malloc(&X, xbytes);
         if (rc == SPTMM_OK) rc = sptmm_malloc(&C, cbytes);
         if (rc == SPTMM_OK) rc = sptmm_memset(X, 0, xbytes);
         if (rc == SPTMM_OK) rc = sptmm_stream_create(&stream);
+        if (rc == SPTMM_OK && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = fail(SPTMM_ERR_HIP, "hipEventCreate");
         if (rc != SPTMM_OK) {
             cleanup();
             return rc;
         }
-        // microseconds per GEMV under `plan`: best of three short loops after a rotation of warm-up
+        std::vector<const void *> xs(per, X);
+        std::vector<void *> cs(per);
+        for (int i = 0; i < per; ++i) cs[i] = (int32_t *)C + (size_t)i * M * w->info.N;
+        // `passes` walks over all the copies: one GEMV per launch, or one batched launch per group of `per`
+        auto walk = [&](int passes) -> int {
+            for (int p = 0; p < passes; ++p)
+                for (int g = 0; g < groups; ++g) {
+                    const int r = batched ? sptmm_gemv_batched(ws.data() + (size_t)g * per, xs.data(), cs.data(), per, M, act, stream)
+                                          : gemv_common(ws[g], X, M, C, stream, (ActType)act);
+                    if (r != SPTMM_OK) return r;
+                }
+            return SPTMM_OK;
+        };
+        // microseconds per GEMV under `plan`: best of three timed loops after a pass of warm-up
         auto time_plan = [&](const Plan &plan, double *us) -> int {
             w->plans[slot] = plan;
             for (sptmm_weights *c : owned) c->plans[slot] = plan;
-            const int iters = batched ? 6 * n : std::max(3 * n, 48);
-            double best = 1e30, t = 0;
-            if (int r = measure_gemv(ws.data(), n, act, X, M, C, batched ? n : n, batched ? 3 : 0, stream, &t)) return r;
+            const int passes = std::max(2, (batched ? 16 : 64) / groups);
+            if (int r = walk(1)) return r;
+            double best = 1e30;
             for (int rep = 0; rep < 3; ++rep) {
-                if (int r = measure_gemv(ws.data(), n, act, X, M, C, iters, batched ? 3 : 0, stream, &t)) return r;
-                best = std::min(best, t);
+                float ms = 0.f;
+                HIP_TRY(hipEventRecord(e0, (hipStream_t)stream));
+                if (int r = walk(passes)) return r;
+                HIP_TRY(hipEventRecord(e1, (hipStream_t)stream));
+                HIP_TRY(hipEventSynchronize(e1));
+                HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+                best = std::min(best, (double)ms * 1000.0 / ((double)passes * n));
             }
             *us = best;
             return SPTMM_OK;
