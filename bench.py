@@ -350,11 +350,11 @@ def run(argv=None):
 
     single = {}
     if "single" in legs:
-        n1 = 4096
+        n1 = a.reps or 4096  # launches per timed loop
         single = {
             "cold_us": round(timed(copies, n1, 256, 0)[0], 3),   # one GEMV per launch, rotating over the copies
             "warm_us": round(timed(copies[:1], n1, 256, 0)[0], 3),  # same stream every launch (reference protocol)
-            "sync_each_call_us": round(timed(copies[:1], 2000, 50, 1)[0], 3),  # + host sync per launch (main.cu:1456)
+            "sync_each_call_us": round(timed(copies[:1], min(n1, 2000), 50, 1)[0], 3),  # + host sync per launch (main.cu:1456)
             # still one GEMV per launch, launch i on stream i % 4: independent GEMVs overlap each other's ramp and tail
             # (best of three: here the host has to issue a launch every 0.8 us, and anything else running on it shows)
             "cold_four_streams_us": round(min(timed(copies, n1, 256, 4)[0] for _ in range(3)), 3),
