@@ -1388,7 +1388,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         }
     }
     if (a.quant) {
-        if constexpr (sizeof(Act) == 1) {
+        if constexpr (sizeof(Act) == 1 && !is_byte_rows<Act>()) {  // (quantising launches never take the byte tile: no such kernels are built)
             auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, true, MERGED>;
             // + room for the per-wavefront sums of a full workgroup, the row maxima and the rows' 1/s
             lds = tile + (size_t)(2 * LISTS_MAX_WAVES + 1) * MT * 4;
