@@ -88,6 +88,11 @@ int sptmm_lists_from_dense(const int8_t *W_colmajor, int K, int N, int S, uint16
 /* Seeded int8 activations, uniform on [-127,127] (stands in for make_X,
  * main.cu:784-797, which is unseeded): xorshift32 stream, r % 255 - 127. */
 int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X);
+/* Seeded ~N(0,1) activations for the float variants (the reference has none: its X is `char` everywhere,
+ * main.cu:784-797): Box-Muller over the same xorshift32 stream, two values per pair of draws
+ * (u1 = (r + 1) / (2^32 + 1), u2 = r / 2^32).  Either output may be NULL: X32 receives the floats, X16 their IEEE
+ * half bits (round to nearest even). */
+int sptmm_make_x_normal(uint32_t seed, size_t count, float *X32, uint16_t *X16);
 
 /* The split_k this library would pick for a balanced matrix (kind: SPTMM_KIND_U16 or
  * SPTMM_KIND_DELTA) on a device with `compute_units` CUs (0: 256) -- what the upload calls use when

@@ -7,7 +7,7 @@ import os
 import numpy as np
 
 __all__ = [
-    "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8",
+    "SptmmError", "lib", "lib_path", "device_init", "generate_ternary", "lists_from_dense", "make_x_i8", "make_x_normal",
     "pack_u16", "unpack_u16", "delta_bits", "pack_delta", "unpack_delta", "pack_i2s", "unpack_i2s", "pack_ragged", "unpack_ragged",
     "generate_ternary_iid", "dense_from_i2s_words", "choose_split_k", "wide_k_tile", "pack_wide", "unpack_wide",
     "i2s_pack_word", "i2s_decode_word", "Weights", "DeviceBuffer", "Stream", "Event", "copy_kernel", "read_kernel",
@@ -22,7 +22,7 @@ _LIB = None
 
 # every symbol include/sptmm.h declares
 EXPORTS = [
-    "sptmm_last_error", "sptmm_version", "sptmm_generate_ternary", "sptmm_lists_from_dense", "sptmm_make_x_i8",
+    "sptmm_last_error", "sptmm_version", "sptmm_generate_ternary", "sptmm_lists_from_dense", "sptmm_make_x_i8", "sptmm_make_x_normal",
     "sptmm_pack_u16_bytes", "sptmm_pack_u16", "sptmm_unpack_u16", "sptmm_delta_bits", "sptmm_pack_delta_bytes",
     "sptmm_pack_delta", "sptmm_unpack_delta", "sptmm_i2s_pack_word", "sptmm_i2s_decode_word",
     "sptmm_pack_i2s_bytes", "sptmm_pack_i2s", "sptmm_unpack_i2s", "sptmm_pack_ragged_bytes", "sptmm_pack_ragged",
@@ -115,6 +115,7 @@ def lib() -> C.CDLL:
         L.sptmm_read_kernel.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
                                         C.POINTER(C.c_double)]
         L.sptmm_make_x_i8.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p]
+        L.sptmm_make_x_normal.argtypes = [C.c_uint32, C.c_size_t, C.c_void_p, C.c_void_p]
         L.sptmm_generate_ternary_iid.argtypes = [C.c_int, C.c_int, C.c_uint32, C.c_double, C.c_double, C.c_void_p]
         for n in ("sptmm_stream_create", "sptmm_event_create"):
             getattr(L, n).argtypes = [C.POINTER(C.c_void_p)]
@@ -178,6 +179,18 @@ def make_x_i8(seed: int, M: int, K: int) -> np.ndarray:
     X = np.empty((M, K), np.int8)
     _ck(lib().sptmm_make_x_i8(seed, M * K, _p(X)))
     return X
+
+
+def make_x_normal(seed: int, M: int, K: int, dtype=np.float16) -> np.ndarray:
+    """Seeded ~N(0,1) activations (Box-Muller over xorshift32), float16 or float32."""
+    if dtype == np.float32:
+        X = np.empty((M, K), np.float32)
+        _ck(lib().sptmm_make_x_normal(seed, M * K, _p(X), None))
+        return X
+    assert dtype == np.float16
+    X = np.empty((M, K), np.uint16)
+    _ck(lib().sptmm_make_x_normal(seed, M * K, None, _p(X)))
+    return X.view(np.float16)
 
 
 def pack_u16(pos, neg, K, split_k) -> np.ndarray:

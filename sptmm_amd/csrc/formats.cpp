@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <array>
 #include <cstdio>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <exception>
@@ -218,6 +219,48 @@ int sptmm_make_x_i8(uint32_t seed, size_t count, int8_t *X)
     if (!X) return fail(SPTMM_ERR_INVALID, "null pointer");
     uint32_t st = seed ? seed : 1u;
     for (size_t i = 0; i < count; ++i) X[i] = (int8_t)((int)(xorshift32(st) % 255u) - 127);
+    return SPTMM_OK;
+}
+
+// float -> IEEE half bits, round to nearest even
+static uint16_t half_bits(float x)
+{
+    uint32_t b;
+    memcpy(&b, &x, 4);
+    const uint32_t sign = (b >> 16) & 0x8000u;
+    const int32_t e = (int32_t)((b >> 23) & 0xff) - 127 + 15;
+    uint32_t m = b & 0x7fffffu;
+    if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign;
+        m |= 0x800000u;
+        const uint32_t shift = (uint32_t)(14 - e);
+        uint32_t h = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (h & 1))) ++h;
+        return (uint16_t)(sign | h);
+    }
+    uint32_t h = ((uint32_t)e << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1))) ++h;
+    return (uint16_t)(sign | h);
+}
+
+int sptmm_make_x_normal(uint32_t seed, size_t count, float *X32, uint16_t *X16)
+{
+    if (!X32 && !X16) return fail(SPTMM_ERR_INVALID, "null pointer");
+    uint32_t st = seed ? seed : 1u;
+    for (size_t i = 0; i < count; i += 2) {
+        const double u1 = (xorshift32(st) + 1.0) / 4294967297.0, u2 = xorshift32(st) / 4294967296.0;
+        const double r = std::sqrt(-2.0 * std::log(u1));
+        const float a = (float)(r * std::cos(6.283185307179586 * u2)), b = (float)(r * std::sin(6.283185307179586 * u2));
+        if (X32) X32[i] = a;
+        if (X16) X16[i] = half_bits(a);
+        if (i + 1 < count) {
+            if (X32) X32[i + 1] = b;
+            if (X16) X16[i + 1] = half_bits(b);
+        }
+    }
     return SPTMM_OK;
 }
 

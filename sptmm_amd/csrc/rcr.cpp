@@ -146,48 +146,6 @@ void parse(int argc, char **argv, Flags &f)
     }
 }
 
-uint32_t xorshift32(uint32_t &s)
-{
-    s ^= s << 13;
-    s ^= s >> 17;
-    s ^= s << 5;
-    return s;
-}
-
-uint16_t float_to_half(float x)
-{
-    uint32_t b;
-    memcpy(&b, &x, 4);
-    uint32_t sign = (b >> 16) & 0x8000u;
-    int32_t e = (int32_t)((b >> 23) & 0xff) - 127 + 15;
-    uint32_t m = b & 0x7fffffu;
-    if (e >= 31) return (uint16_t)(sign | 0x7c00u);
-    if (e <= 0) {
-        if (e < -10) return (uint16_t)sign;
-        m |= 0x800000u;
-        uint32_t shift = (uint32_t)(14 - e);
-        uint32_t h = m >> shift, rem = m & ((1u << shift) - 1), halfway = 1u << (shift - 1);
-        if (rem > halfway || (rem == halfway && (h & 1))) ++h;
-        return (uint16_t)(sign | h);
-    }
-    uint32_t h = ((uint32_t)e << 10) | (m >> 13), rem = m & 0x1fffu;
-    if (rem > 0x1000u || (rem == 0x1000u && (h & 1))) ++h;
-    return (uint16_t)(sign | h);
-}
-
-// ~N(0,1) from the same xorshift stream (Box-Muller)
-void make_x_normal(uint32_t seed, size_t n, std::vector<float> &out)
-{
-    uint32_t st = seed ? seed : 1u;
-    out.resize(n);
-    for (size_t i = 0; i < n; i += 2) {
-        double u1 = (xorshift32(st) + 1.0) / 4294967297.0, u2 = xorshift32(st) / 4294967296.0;
-        double r = std::sqrt(-2.0 * std::log(u1));
-        out[i] = (float)(r * std::cos(6.283185307179586 * u2));
-        if (i + 1 < n) out[i + 1] = (float)(r * std::sin(6.283185307179586 * u2));
-    }
-}
-
 float half_to_float(uint16_t h)
 {
     const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
@@ -362,12 +320,8 @@ int main(int argc, char **argv)
     if (act == 0) {
         CHECK_SPTMM(sptmm_make_x_i8(seed, xcount, (int8_t *)xhost.data()));
     } else {
-        std::vector<float> xf;
-        make_x_normal(seed, xcount, xf);
-        if (act == 2)
-            memcpy(xhost.data(), xf.data(), xcount * 4);
-        else
-            for (size_t i = 0; i < xcount; ++i) ((uint16_t *)xhost.data())[i] = float_to_half(xf[i]);
+        // ~N(0,1), Box-Muller over the same seeded stream
+        CHECK_SPTMM(sptmm_make_x_normal(seed, xcount, act == 2 ? (float *)xhost.data() : nullptr, act == 1 ? (uint16_t *)xhost.data() : nullptr));
     }
 
     // The host's own result: the reference kernel's gather-sum over the lists this process holds (exact int32 for int8

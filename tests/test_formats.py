@@ -386,3 +386,32 @@ def test_automatic_split_k_is_valid_and_follows_the_measured_rule():
     for bad in ((sp.KIND_I2S, 64, 64), (sp.KIND_U16, 0, 64), (sp.KIND_U16, 64, 0), (sp.KIND_U16, 64, 31), (sp.KIND_U16, -16, 64)):
         with pytest.raises(sp.SptmmError):
             sp.choose_split_k(*bad)
+
+
+def test_seeded_normal_activations_are_box_muller_over_xorshift32():
+    """sptmm_make_x_normal against the same recipe in numpy / Python: pairs (u1, u2) from consecutive xorshift32 draws,
+    r = sqrt(-2 ln u1), values r cos(2 pi u2), r sin(2 pi u2); the fp16 output is the fp32 one rounded to nearest even."""
+    import math
+
+    def xs(s):
+        s ^= (s << 13) & 0xFFFFFFFF
+        s ^= s >> 17
+        s ^= (s << 5) & 0xFFFFFFFF
+        return s
+
+    seed, n = 0xC0FFEE ^ 3, 41
+    st, want = seed, []
+    while len(want) < n:
+        st = xs(st)
+        u1 = (st + 1.0) / 4294967297.0
+        st = xs(st)
+        u2 = st / 4294967296.0
+        r = math.sqrt(-2.0 * math.log(u1))
+        want += [r * math.cos(6.283185307179586 * u2), r * math.sin(6.283185307179586 * u2)]
+    want = np.array(want[:n], np.float64)
+    x32 = sp.make_x_normal(seed, 1, n, np.float32)[0]
+    x16 = sp.make_x_normal(seed, 1, n, np.float16)[0]
+    assert np.allclose(x32, want, rtol=1e-6, atol=1e-7)
+    assert (x16 == x32.astype(np.float16)).all()
+    big = sp.make_x_normal(7, 64, 4096, np.float32)
+    assert abs(big.mean()) < 0.01 and abs(big.std() - 1.0) < 0.01

@@ -767,3 +767,35 @@ def test_gap_stream_four_rows_single_launch_with_several_tasks_per_wavefront():
             X = x_i8(77 + M, M, K)
             assert (w.matmul(X) == oracle.sptmm_i8_mt(X, pos, neg, 8)).all(), (split, M)
         w.free()
+
+
+@pytest.mark.parametrize("M", [5, 8, 9, 13])
+def test_fp32_rows_beyond_one_four_row_tile(M):
+    """fp32 rows are summed in tiles of four (a 16-byte slot per index): M above four takes several tiles in one launch
+    (the grid's second dimension), the last one partly empty.  u16 lists, both gap widths, a ragged matrix, alone and
+    batched, against the float64 gather-sum within 1e-3 of max(|ref|, sqrt(S))."""
+    K, N, S = 2560, 640, 1536
+    W, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    X = oracle.make_x_normal(50 + M, M, K, np.float32)
+    ref = oracle.sptmm_f64(X, pos, neg)
+    for name, w in (("u16", sp.Weights.upload_u16(pos, neg, K, 32)), ("u16 split 128", sp.Weights.upload_u16(pos, neg, K, 128)),
+                    ("gaps", sp.Weights.upload_delta(pos, neg, K, 16)), ("ragged u16", sp.Weights.upload_dense(W, sp.KIND_U16, 32)),
+                    ("ragged gaps", sp.Weights.upload_dense(W, sp.KIND_DELTA, 8))):
+        say("fp32 rows", name, "M", M)
+        check_fp(w.matmul(X), ref, S)
+        xb = [sp.DeviceBuffer.from_numpy(X) for _ in range(3)]
+        cb = [sp.DeviceBuffer(4 * M * N) for _ in range(3)]
+        cl = [w, w.clone(), w.clone()]
+        sp.gemv_batched(cl, xb, cb, M, 2)
+        sp.device_sync()
+        for c in cb:
+            check_fp(c.to_numpy(np.float32, (M, N)), ref, S)
+        for o in xb + cb + cl:
+            o.free()
+    # 16-bit gaps (a matrix too sparse for byte gaps, balanced lists)
+    Ks, Ns, Ss = 6912, 64, 256
+    _, ps, ns = sp.generate_ternary(Ks, Ns, Ss)
+    Xs = oracle.make_x_normal(9, M, Ks, np.float32)
+    w = sp.Weights.upload_delta(ps, ns, Ks, 8)
+    check_fp(w.matmul(Xs), oracle.sptmm_f64(Xs, ps, ns), Ss)
+    w.free()
