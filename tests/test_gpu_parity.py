@@ -792,7 +792,7 @@ def test_fp32_rows_beyond_one_four_row_tile(M):
             check_fp(c.to_numpy(np.float32, (M, N)), ref, S)
         for o in xb + cb + cl:
             o.free()
-    # 16-bit gaps (a matrix too sparse for byte gaps, balanced lists)
+    # a matrix too sparse for plain byte gaps (balanced lists: the stream walks long gaps over zero slots, or takes 16-bit gaps)
     Ks, Ns, Ss = 6912, 64, 256
     _, ps, ns = sp.generate_ternary(Ks, Ns, Ss)
     Xs = oracle.make_x_normal(9, M, Ks, np.float32)
