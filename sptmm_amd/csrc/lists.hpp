@@ -1288,7 +1288,12 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // (also where two tiles would fit a compute unit: the registers of an eight-row kernel allow 16 wavefronts per CU either
     // way, and one workgroup of 16 stages the tile once -- K=6912 N=2560, M=8, 8 -> 16 wavefronts: u16 3.65 -> 3.40 us, gap
     // stream level at 2.14-2.40 us from box to box)
-    if (MT == 8 && a.batch >= 4 && a.W == 1 && !a.quant) wpb = lists_max_waves<Act, MT, false>() / 4 * 4;
+    if (MT == 8 && a.batch >= 4 && a.W == 1 && !a.quant) {
+        wpb = lists_max_waves<Act, MT, false>() / 4 * 4;
+        // ... as long as the launch still has two workgroups per compute unit: a narrow matrix takes smaller ones
+        // (K=12800 N=256, 64 tasks, 16 GEMVs per launch: 16 -> 4 wavefronts 1.43 -> 0.95 us per GEMV; K=6656 N=512: 0.78 -> 0.62)
+        while (wpb > 4 && (long)a.batch * ((a.tasks + wpb - 1) / wpb) < 2L * cus) wpb -= 4;
+    }
     // four-row tiles on gap streams, batched, tile small enough for several workgroups per CU: four wavefronts for
     // int8 rows (K=2560 N=640 0.32 -> 0.29 us per GEMV, M=2 on the headline shape 1.76 -> 1.67; level elsewhere), eight
     // for fp16 rows (headline shape 57 -> 64 % of HBM peak, K=2560 N=6912 61 -> 66 %; with the 55 KB tile of K=13824
@@ -1305,6 +1310,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // wavefront by the search below (headline shape, 32 GEMVs: 5 wavefronts x 2 tasks 6.75 us per GEMV, 8 x 4 4.10,
     // 8 x 10 -- two full rounds -- 3.73 us = 71 % of HBM peak; gap stream 4.13 -> 3.46 us)
     if (MT == 4 && sizeof(Act) == 4 && a.batch >= 4 && a.W == 1) wpb = max_waves;
+    // tiles of 32 KB or more under anything but the one-row int8 kernels: eight wavefronts, and tasks per wavefront by the
+    // search below (the kernels with rules of their own above keep their workgroup size)
+    const bool big_tile = tile >= 32 * 1024 && !(MT == 1 && sizeof(Act) == 1) && a.batch >= 4 && a.W == 1 && !a.quant;
+    if (big_tile && MT != 8 && !(MT == 4 && sizeof(Act) == 4) && !(MT == 4 && MODE != 0 && sizeof(Act) == 1)) wpb = std::min(8, max_waves);
     if (tune_wpb > 0 && tune_wpb <= (a.quant ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>()) && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
@@ -1316,7 +1325,11 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // pays for staging the tile: two tasks per wavefront halve that (measured: gap streams 1.88 -> 1.72 us
     // per GEMV, four-row tiles 2.83 -> 2.76; nothing for the one-row u16 kernel, which waits on HBM only).
     constexpr bool WIDE_SLOT = MT == 8 || (MT == 4 && sizeof(Act) == 4);  // 16 bytes per index
-    if ((WIDE_SLOT || (MT == 4 && MODE != 0)) && a.batch >= 4 && wgs == 1) {
+    // ... and so is any tile of 32 KB or more, whatever the rows (float rows at K=13824, 32 GEMVs per launch, two tasks per
+    // wavefront -> this search: gap stream fp16 M=1 8.3 -> 6.45 us per GEMV, fp32 M=4 32.0 -> 22.4; u16 lists fp16 M=4
+    // 17.6 -> 12.7, fp32 M=4 52 -> 36; int8 M=4 on u16 lists at K=11008-13568 7.3 -> 6.5 and 9.0 -> 8.3) -- except under
+    // the one-row int8 kernels, which wait on HBM alone and do best with one task per wavefront up to 55 KB tiles.
+    if ((WIDE_SLOT || (MT == 4 && MODE != 0) || big_tile) && a.batch >= 4 && wgs == 1) {
         // Multi-row tiles are expensive to stage (eight rows of K=13824: 110 KB, ~2.5 us against ~4 us per task) and their
         // walks are bound by the LDS and the matrix unit rather than by HBM: up to 16 tasks per wavefront, chosen so that the
         // launch's workgroups come in full rounds over the workgroups the chip holds at once (cost per round: staging

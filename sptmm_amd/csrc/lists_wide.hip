@@ -399,6 +399,16 @@ static int launch_wide_v(const GemvArgs &a, const WideHeader &h, hipStream_t st)
     // 16 wavefronts: u16 15.9 -> 15.4 us per GEMV, gap stream 14.2 -> 12.7 us; a lone u16 GEMV 27.9 -> 24.4 us HBM-cold
     // on 160 of the 256 compute units, a lone gap-stream GEMV 23.8 -> 24.4 us, so that one keeps the smaller workgroups)
     if ((a.batch >= 4 || MODE == 0) && wpb >= 8) wpb = MAXW / per_cu;  // (shapes with tasks enough to fill the chip that way)
+    // A batched launch takes the largest workgroup whatever its task count: it fills the chip along blockIdx.z, and a
+    // workgroup of four wavefronts staged a whole tile for four tasks (8 GEMVs per launch, 16 rows: K=5376 N=3840 S=2016
+    // 4 -> 16 wavefronts gap stream 6.04 -> 2.66 us per GEMV, u16 4.69 -> 3.05; K=9728 N=6400 S=512 u16 2.71 -> 1.96;
+    // K=2048 N=3840 S=1088, two tiles per compute unit, 4 -> 8: 2.62 -> 1.87)
+    if (a.batch >= 4) {
+        wpb = MAXW / per_cu;
+        // (as long as its workgroups cover three quarters of the compute units: K=12800 N=256, 8 GEMVs of 64 tasks: 16 -> 8
+        // wavefronts 2.47 -> 1.90 us per GEMV, K=6656 N=512 1.51 -> 1.09; K=6912 N=1792, 224 workgroups of 16, is best left so)
+        while (wpb > 8 && (long)a.batch * ((a.tasks + wpb - 1) / wpb) * 4 < 3L * cus * per_cu) wpb -= 4;
+    }
     if (tune_wpb > 0 && tune_wpb <= MAXW) wpb = tune_wpb;
     const int blocks = (a.tasks + wpb - 1) / wpb;
     int grid_x = blocks < cus * per_cu ? blocks : cus * per_cu;
