@@ -415,8 +415,20 @@ static int launch_i2s_mfma(const GemvArgs &a, hipStream_t st)
         // ... as long as the launch still has workgroups enough: four per compute unit, eight where a workgroup's share
         // of K is short (K=2560, 32 GEMVs per launch: N=640 4 -> 1 tiles 0.200 -> 0.154 us per GEMV, N=2560 4 -> 2 tiles
         // 0.379 -> 0.355 us; N=6912 stays at 4: 0.82 against 0.89 / 1.05 us)
-        const long need = (long)(a.compute_units > 0 ? a.compute_units : 256) * (rounds >= 16 ? 4 : 8);
-        while (ct > 1 && (long)a.batch * (groups / ct) < need) ct /= 2;
+        const long cus = a.compute_units > 0 ? a.compute_units : 256;
+        if (xj >= 3) {
+            // Nine rows and more: the reuse of X counts for more than the number of workgroups.  Short K goes to two
+            // wavefronts per workgroup, and tiles are given up only while the launch has fewer than six wavefronts per
+            // compute unit (32 GEMVs of 16 rows per launch, (tiles, wavefronts) -> us per GEMV: K=2560 N=2560 (2,4) 0.59,
+            // (4,2) 0.43; K=2560 N=3840 (4,4) 0.84 as chosen before, (8,2) 0.59; K=6912 N=2560 (8,4) 0.92, (4,2) 0.89;
+            // K=4096 N=4096 (8,4) 0.87, (8,2) 0.82; K=13824 N=5120 stays at (8,4): 2.99 against 3.12 for (8,2))
+            waves = rounds >= 40 ? 4 : 2;
+            while (ct > 1 && (long)a.batch * (groups / ct) * waves < 6 * cus) ct /= 2;
+            if (ct == 1) waves = 4;
+        } else {
+            const long need = cus * (rounds >= 16 ? 4 : 8);
+            while (ct > 1 && (long)a.batch * (groups / ct) < need) ct /= 2;
+        }
     } else {
         while (ct < 4 && groups / (2 * ct) >= 160) ct *= 2;
     }
