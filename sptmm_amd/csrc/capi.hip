@@ -776,12 +776,18 @@ int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_m
                 if (rc == SPTMM_OK && t < t_best) t_best = t, best = p;
             }
         if (rc == SPTMM_OK) {
-            // the model's shape stays unless the search found something at least 2 % faster, confirmed by a second timing
+            // The model's shape stays unless the search found something at least 2 % faster, and still is when both are timed
+            // again side by side: the model's first timing is the first work the search puts on the device, and on its own it
+            // read up to a tenth slow (the same shape "found" again as a plan the launcher ignores: 3.83 against 3.40 us).
             if (t_best < 0.98 * t_model) {
-                double again = 0;
-                rc = time_plan(best, &again);
-                if (rc == SPTMM_OK && again >= 0.98 * t_model) best = Plan{}, t_best = t_model;
-                else if (rc == SPTMM_OK) t_best = std::min(t_best, again);
+                double model_again = 0, again = 0;
+                rc = time_plan(Plan{}, &model_again);
+                if (rc == SPTMM_OK) rc = time_plan(best, &again);
+                if (rc == SPTMM_OK) {
+                    t_model = std::min(t_model, model_again);
+                    if (again >= 0.98 * t_model) best = Plan{}, t_best = t_model;
+                    else t_best = std::min(t_best, again);
+                }
             } else {
                 best = Plan{}, t_best = t_model;
             }

@@ -1314,6 +1314,10 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     // search below (the kernels with rules of their own above keep their workgroup size)
     const bool big_tile = tile >= 32 * 1024 && !(MT == 1 && sizeof(Act) == 1) && a.batch >= 4 && a.W == 1 && !a.quant;
     if (big_tile && MT != 8 && !(MT == 4 && sizeof(Act) == 4) && !(MT == 4 && MODE != 0 && sizeof(Act) == 1)) wpb = std::min(8, max_waves);
+    // eight fp16 rows, batched, three tiles or more to a compute unit: workgroups of four wavefronts, with the tasks per
+    // wavefront the search below gives them (32 GEMVs per launch, K=2560: N=6912 gap stream 4.09 -> 3.39 us per GEMV,
+    // N=13824 7.81 -> 6.46 and u16 lists 8.64 -> 7.43, N=3840 2.25 -> 1.95 and 2.29 -> 2.11; K=4096, two tiles: eight stay ahead)
+    if (MT == 8 && sizeof(Act) == 2 && a.batch >= 4 && a.W == 1 && !a.quant && 3 * (tile + lists_behind_tile<Act, MT>(4)) <= (size_t)a.lds_limit) wpb = 4;
     if (tune_wpb > 0 && tune_wpb <= (a.quant ? LISTS_MAX_WAVES : lists_max_waves<Act, MT, false>()) && tune_wpb % a.W == 0) wpb = tune_wpb;
     const int slots = cus * wgs;  // workgroups resident at once
     const int blocks = (a.tasks + wpb - 1) / wpb;
