@@ -1248,12 +1248,16 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             const int blocks = (a.tasks + w - 1) / w;
             const int grid = blocks < cus * g ? blocks : cus * g;
             const int iters = (blocks + grid - 1) / grid;
-            const double r = (double)g * w;
+            // tasks a compute unit has in flight: in the full passes, and in the last one, which the workgroups may not fill
+            const double r = std::min((double)g * w, (double)grid * w / cus);
+            const int full = blocks / grid, rest = blocks - full * grid;
+            const double r_rest = (double)rest * w / cus;
             // + each workgroup stages the tile once; a bubble per extra pass; when latency-bound, spread over more CUs
             // (where the latency term leaves several workgroup sizes level, four or five wavefronts: a lone launch of few
             // tasks does better in a few such workgroups than in one or two wavefronts on every compute unit -- K=4352
             // N=512 S=992, 128 tasks: 3.64 -> 3.20 us in workgroups of five; K=6400 N=2048 S=1952, gap stream: 4.39 -> 3.94)
-            const double cost = iters * (r > r_lat ? r : r_lat) + 0.05 * g + 0.25 * (iters - 1) + 0.001 * (w < 4 ? 4.5 - w : w - 4.5);
+            const double cost = full * (r > r_lat ? r : r_lat) + (rest ? (r_rest > r_lat ? r_rest : r_lat) : 0.0) + 0.05 * g + 0.25 * (iters - 1) +
+                                0.001 * (w < 4 ? 4.5 - w : w - 4.5);
             if (cost < best - 1e-9) {
                 best = cost;
                 wpb = w;
