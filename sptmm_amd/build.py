@@ -58,7 +58,7 @@ def build_rcr() -> str:
     if not os.path.exists(src):
         return ""
     _run(["g++", "-O2", "-std=c++17", "-Wall", "-o", RCR, src, "-L" + PKG, "-lsptmm",
-          "-Wl,-rpath,$ORIGIN/..", "-pthread"])
+          "-Wl,-rpath,$ORIGIN/..", "-pthread", "-ldl"])
     return RCR
 
 

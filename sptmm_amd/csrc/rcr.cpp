@@ -13,7 +13,8 @@
 // same lists computed here on the host ("# check=PASS"), and that host loop is
 // timed on the cores this process may use ("# cpu: ...").  -cpu_only runs the
 // host side alone (no device needed): the CPU line, and the gather-sum checked
-// against the plain dense product of the same matrix.
+// against the plain dense product of the same matrix.  -cu_blas runs the dense
+// int8 product of the same matrix through rocBLAS, loaded when the flag is given.
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -27,6 +28,7 @@
 #include <thread>
 #include <vector>
 
+#include <dlfcn.h>
 #include <sched.h>
 
 #include "../../include/sptmm.h"
@@ -272,6 +274,49 @@ void host_dense_product(const T *X, int M, int K, int N, const int8_t *W, int th
     });
 }
 
+// The dense int8 product through rocBLAS, loaded at run time (no link-time dependency): what main.cu:842-873 asks of
+// cuBLAS, in the layouts this build has -- X row-major [M][K], W column-major [K][N], C row-major [M][N], which in the
+// library's column-major terms is C^T [N x M] = W^T [N x K] * X^T [K x M].  (The reference's own line only runs in an
+// all-column-major build and passes a null weight pointer, main.cu:836, 863.)
+struct DenseBlas {
+    typedef int (*create_fn)(void **);
+    typedef int (*destroy_fn)(void *);
+    typedef int (*set_stream_fn)(void *, void *);
+    typedef int (*gemm_ex_fn)(void *, int, int, int, int, int, const void *, const void *, int, int, const void *, int, int, const void *,
+                              const void *, int, int, void *, int, int, int, int, int32_t, uint32_t);
+    void *so = nullptr, *handle = nullptr;
+    create_fn create = nullptr;
+    destroy_fn destroy = nullptr;
+    set_stream_fn set_stream = nullptr;
+    gemm_ex_fn gemm_ex = nullptr;
+
+    bool open(void *stream, std::string *why)
+    {
+        for (const char *name : {"librocblas.so.5", "librocblas.so", "/opt/rocm/lib/librocblas.so"})
+            if ((so = dlopen(name, RTLD_NOW | RTLD_LOCAL))) break;
+        if (!so) return *why = std::string("cannot load rocBLAS: ") + dlerror(), false;
+        create = (create_fn)dlsym(so, "rocblas_create_handle");
+        destroy = (destroy_fn)dlsym(so, "rocblas_destroy_handle");
+        set_stream = (set_stream_fn)dlsym(so, "rocblas_set_stream");
+        gemm_ex = (gemm_ex_fn)dlsym(so, "rocblas_gemm_ex");
+        if (!create || !destroy || !set_stream || !gemm_ex) return *why = "rocBLAS lacks rocblas_gemm_ex", false;
+        if (int rc = create(&handle)) return *why = "rocblas_create_handle: status " + std::to_string(rc), false;
+        if (int rc = set_stream(handle, stream)) return *why = "rocblas_set_stream: status " + std::to_string(rc), false;
+        return true;
+    }
+    // rocblas_operation_transpose = 112, _none = 111; rocblas_datatype_i8_r = 160, _i32_r = 162; rocblas_gemm_algo_standard = 0
+    int product(const void *W_d, const void *X_d, void *C_d, int M, int K, int N) const
+    {
+        const int32_t alpha = 1, beta = 0;
+        return gemm_ex(handle, 112, 111, N, M, K, &alpha, W_d, 160, K, X_d, 160, K, &beta, C_d, 162, N, C_d, 162, N, 162, 0, 0, 0);
+    }
+    void close()
+    {
+        if (handle) destroy(handle);
+        handle = nullptr;
+    }
+};
+
 struct Method {
     const char *label;
     sptmm_weights *w;
@@ -289,7 +334,7 @@ int main(int argc, char **argv)
                "  -row_split3_small <splitK>  SpTMM over u16 index lists (8,16,32,64,128,256)\n"
                "  -row_split_delta2 <splitK>  SpTMM-delta over 8/16-bit gap streams (8,16,32,64)\n"
                "  -i2s                        2-bit packed dense-ternary baseline\n"
-               "  -cu_blas                    not available in this layout (aborts like the reference's rcr)\n"
+               "  -cu_blas                    the dense int8 product of the same matrix through rocBLAS (loaded at run time)\n"
                "  -M -K -N -S -L -iter        shape, nonzeros per column, iterations\n"
                "  -act i8|f16|f32  -seed <n>  -cold <copies>  -nocheck  -nocpu (no host timing)\n"
                "  -cpu_only                   host side only: CPU line and the lists checked against the dense product\n");
@@ -301,13 +346,13 @@ int main(int argc, char **argv)
     if (f.M < 1 || f.M > (1u << 20)) strict_fail("M out of range");
 
     // host side first (needs no GPU): shape rules of main.cu:85-91 and the seeded ternary matrix
-    const bool any = f.row_split3_small || f.row_split_delta2 || f.i2s;
+    const bool any = f.row_split3_small || f.row_split_delta2 || f.i2s || f.cu_blas;
     std::vector<uint16_t> pos, neg;
     std::vector<int8_t> dense;
     if (any) {
         pos.resize((size_t)N * (size_t)std::max(S / 2, 0));
         neg.resize(pos.size());
-        if ((f.i2s || f.cpu_only) && K > 0 && N > 0) dense.resize((size_t)K * N);
+        if ((f.i2s || f.cu_blas || f.cpu_only) && K > 0 && N > 0) dense.resize((size_t)K * N);
         CHECK_SPTMM(sptmm_generate_ternary(K, N, S, dense.empty() ? nullptr : dense.data(), pos.data(), neg.data()));
         if (f.row_split3_small && !sptmm_pack_u16_bytes(N, S, (int)f.row_split3_small)) strict_fail("Wrong split size");
         if (f.row_split_delta2 && !sptmm_pack_delta_bytes(N, S, (int)f.row_split_delta2, 8)) strict_fail("Wrong split size");
@@ -408,9 +453,62 @@ int main(int argc, char **argv)
     CHECK_SPTMM(sptmm_stream_create(&stream));
     banner();
 
-    if (f.cu_blas) strict_fail("Wrong layout");  // main.cu:843: the row/col/row build refuses cuBLAS
-
     std::vector<Method> done;
+    if (f.cu_blas) {
+        // first of the methods, as at main.cu:841
+        if (act != 0) strict_fail("cu_blas takes int8 activations");
+        DenseBlas blas;
+        std::string why;
+        if (!blas.open(stream, &why)) {
+            fprintf(stderr, "%s\n", why.c_str());
+            exit(EXIT_FAILURE);
+        }
+        void *w_d = nullptr, *e0 = nullptr, *e1 = nullptr;
+        CHECK_SPTMM(sptmm_malloc(&w_d, dense.size()));
+        CHECK_SPTMM(sptmm_memcpy_h2d(w_d, dense.data(), dense.size()));
+        CHECK_SPTMM(sptmm_event_create(&e0));
+        CHECK_SPTMM(sptmm_event_create(&e1));
+        auto call = [&] {
+            if (int rc = blas.product(w_d, x_d, c_d, M, K, N)) {
+                fprintf(stderr, "rocblas_gemm_ex: status %d (int8 x int8 -> int32, m=%d n=%d k=%d)\n", rc, N, M, K);
+                exit(EXIT_FAILURE);
+            }
+        };
+        CHECK_SPTMM(sptmm_memset(c_d, 0xff, sizeof(int) * (size_t)M * N));
+        for (int i = 0; i < 3; ++i) call();  // (the first call loads the library's kernels)
+        CHECK_SPTMM(sptmm_stream_sync(stream));
+        Method m{"cu_blas", nullptr, std::vector<unsigned char>(sizeof(int) * (size_t)M * N)};
+        CHECK_SPTMM(sptmm_memcpy_d2h(m.result.data(), c_d, m.result.size()));
+        const int iters = (int)std::max<uint32_t>(f.iter, 1);
+        double us_sync = 0, us_b2b = 0;
+        // reference protocol: call + synchronize per iteration (main.cu:852-869)
+        CHECK_SPTMM(sptmm_event_record(e0, stream));
+        for (int i = 0; i < iters; ++i) {
+            call();
+            CHECK_SPTMM(sptmm_stream_sync(stream));
+        }
+        CHECK_SPTMM(sptmm_event_record(e1, stream));
+        CHECK_SPTMM(sptmm_event_sync(e1));
+        CHECK_SPTMM(sptmm_event_elapsed_us(e0, e1, &us_sync));
+        // (printf: libraries loaded at run time may have changed std::cout's precision; %g is what the stream prints by default)
+        printf("%g\n", (double)(float)(us_sync / iters / 1000.0));
+        fflush(stdout);
+        CHECK_SPTMM(sptmm_event_record(e0, stream));
+        for (int i = 0; i < iters; ++i) call();
+        CHECK_SPTMM(sptmm_event_record(e1, stream));
+        CHECK_SPTMM(sptmm_event_sync(e1));
+        CHECK_SPTMM(sptmm_event_elapsed_us(e0, e1, &us_b2b));
+        const double bytes = (double)K * N + (double)M * K + 4.0 * M * N;
+        printf("# cu_blas: us/call sync_each=%.3f back_to_back=%.3f (%.1f GB/s, %.1f%% of %.0f) bytes=%.0f rocBLAS int8 x int8 -> int32, dense\n",
+               us_sync / iters, us_b2b / iters, bytes / (us_b2b / iters) / 1e3, bytes / (us_b2b / iters) / 1e3 / dev.peak_hbm_gbps * 100.0,
+               dev.peak_hbm_gbps, bytes);
+        done.push_back(std::move(m));
+        blas.close();
+        sptmm_event_destroy(e0);
+        sptmm_event_destroy(e1);
+        sptmm_free(w_d);
+    }
+
     auto run = [&](const char *label, sptmm_weights *w, bool timed) {
         sptmm_winfo wi;
         CHECK_SPTMM(sptmm_weights_info(w, &wi));
@@ -433,7 +531,8 @@ int main(int argc, char **argv)
             const sptmm_weights *one[1] = {w};
             // reference protocol: launch + synchronize per iteration (main.cu:1456)
             CHECK_SPTMM(sptmm_measure_gemv(one, 1, a, x_d, M, c_d, iters, 1, stream, &us_sync));
-            std::cout << (float)(us_sync / 1000.0) << std::endl;
+            printf("%g\n", (double)(float)(us_sync / 1000.0));
+            fflush(stdout);
             const int warm = std::min(iters, 200);
             CHECK_SPTMM(sptmm_measure_gemv(one, 1, a, x_d, M, c_d, warm, 0, stream, &us_b2b));
             CHECK_SPTMM(sptmm_measure_gemv(one, 1, a, x_d, M, c_d, iters, 0, stream, &us_b2b));

@@ -149,5 +149,19 @@ def test_float_activations_and_cublas_refusal():
     assert r.returncode == 0 and "# check=PASS (sptmm ~ host; sptmm-delta ~ host; max rel diff" in r.stdout, r.stdout + r.stderr
     r = rcr("-row_split3_small", "32", "-M=2", "-K=512", "-N=64", "-S=128", "-iter=20", "-nocpu")
     assert r.returncode == 0 and "# cpu:" not in r.stdout and "# check=PASS (sptmm == host)" in r.stdout, r.stdout + r.stderr
-    r = rcr("-cu_blas", "-M=1", "-K=6912", "-N=2560", "-S=4096")
-    assert r.returncode == -signal.SIGABRT and "Wrong layout" in r.stderr  # main.cu:843 in the row/col/row build
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_cu_blas_runs_the_dense_product_of_the_same_matrix(M):
+    """-cu_blas (main.cu:842-873): the dense int8 product through rocBLAS, first of the methods as in the reference, its
+    int32 result compared with the host's gather-sum like every other method's."""
+    r = rcr("-cu_blas", "-row_split3_small", "32", "-i2s", "-M=%d" % M, "-K=6912", "-N=2560", "-S=4096", "-iter=50", timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    check_output(r.stdout, 3, M, 6912, 2560, 4096, 50)
+    lines = r.stdout.splitlines()
+    first_comment = [l for l in lines if l.startswith("# ") and "us/call sync_each" in l][0]
+    assert first_comment.startswith("# cu_blas:") and "rocBLAS int8 x int8 -> int32" in first_comment
+    assert "cu_blas == host" in [l for l in lines if l.startswith("# check=")][0]
+    r = rcr("-cu_blas", "-M=1", "-K=6912", "-N=2560", "-S=4096", "-act", "f16")
+    assert r.returncode == -signal.SIGABRT and "int8 activations" in r.stderr
