@@ -240,7 +240,8 @@ size_t sptmm_weights_bytes(const sptmm_weights *w);
  *   rotate over enough device copies of the stream to exceed the last-level cache (`batch` = 0 times lone launches, else launches of `batch`
  *   GEMVs; act as in sptmm_gemv_batched; int8, fp16 or fp32 rows of zeros) -- which stores the fastest as the stream's
  *   plan for that kind of call and reports microseconds per GEMV under the model's shape and under the plan kept (the
- *   model's shape is kept unless a candidate is at least 2 % faster).  Synchronous; allocates and frees its own buffers.
+ *   model's shape is kept unless a candidate is at least 2 % faster, and still is when both are timed again one
+ *   after the other).  Synchronous; allocates and frees its own buffers.
  * Plans travel with sptmm_weights_save / _load and are copied by sptmm_weights_clone. */
 typedef struct sptmm_plan {
     int waves_per_wg;    /* wavefronts per workgroup */
