@@ -233,7 +233,8 @@ size_t sptmm_weights_bytes(const sptmm_weights *w);
 
 /* Launch plans.  The shape of a launch (wavefronts per workgroup, workgroups per compute unit, tasks per wavefront, ...)
  * comes from a model inside the library; a stream may carry its own choice per kind of call -- by activation rows
- * (1, 2-4, 5-8, more) and by lone or batched launch -- which then replaces the model's for that stream.  Every field
+ * (1, 2-4, 5-8, more) and by lone or batched launch, whatever the activation type: tune with the type the stream will
+ * meet -- which then replaces the model's for that stream.  Every field
  * 0 = the model's choice; a value the kernels cannot take is ignored, never an error, and no plan changes a result.
  * The reference fixes its launch shapes at compile time (grid and block per instantiation, main.cu:996-1455).
  *   sptmm_weights_tune: a bounded search on the device -- a few dozen candidate plans, each timed over launches that
