@@ -239,7 +239,7 @@ size_t sptmm_weights_bytes(const sptmm_weights *w);
  * The reference fixes its launch shapes at compile time (grid and block per instantiation, main.cu:996-1455).
  *   sptmm_weights_tune: a bounded search on the device -- a few dozen candidate plans, each timed over launches that
  *   rotate over enough device copies of the stream to exceed the last-level cache (`batch` = 0 times lone launches, else launches of `batch`
- *   GEMVs; act as in sptmm_gemv_batched; int8, fp16 or fp32 rows of zeros) -- which stores the fastest as the stream's
+ *   GEMVs; act as in sptmm_gemv_batched, or 3 / 4 for lone sptmm_gemv_q8 calls on fp16 / bf16 rows; the rows are zeros) -- which stores the fastest as the stream's
  *   plan for that kind of call and reports microseconds per GEMV under the model's shape and under the plan kept (the
  *   model's shape is kept unless a candidate is at least 2 % faster, and still is when both are timed again one
  *   after the other).  Synchronous; allocates and frees its own buffers.

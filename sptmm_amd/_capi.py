@@ -582,7 +582,8 @@ class Weights:
 
     def tune(self, M: int, batch: int = 0, act: int = 0):
         """Bounded on-device search for the launch shape of calls with M rows (batch = 0: lone launches, else launches of
-        `batch` GEMVs); the fastest plan is stored in the object.  -> (us per GEMV with the model's shape, with the plan kept, plan)."""
+        `batch` GEMVs; act 0 int8, 1 fp16, 2 fp32 rows, 3 / 4 the lone quantising call on fp16 / bf16 rows); the fastest plan is
+        stored in the object.  -> (us per GEMV with the model's shape, with the plan kept, plan)."""
         a, b = C.c_double(), C.c_double()
         _ck(lib().sptmm_weights_tune(self.handle, M, batch, act, C.byref(a), C.byref(b)))
         return a.value, b.value, self.get_plan(M, batch > 0)

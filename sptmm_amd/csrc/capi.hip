@@ -673,7 +673,11 @@ int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_m
     return guarded([&]() -> int {
         if (!w) return fail(SPTMM_ERR_INVALID, "null pointer");
         if (M < 1 || batch < 0) return fail(SPTMM_ERR_INVALID, "M must be at least 1 and batch at least 0");
-        if (act < ACT_I8 || act > ACT_F32) return fail(SPTMM_ERR_INVALID, "act must be 0 (int8), 1 (fp16) or 2 (fp32)");
+        // act 3 / 4: the quantising GEMV on fp16 / bf16 rows (sptmm_gemv_q8), lone launches on ordinary streams
+        const bool q8 = act == 3 || act == 4;
+        if ((act < ACT_I8 || act > ACT_F32) && !q8) return fail(SPTMM_ERR_INVALID, "act must be 0 (int8), 1 (fp16), 2 (fp32), 3 or 4 (fp16 / bf16 rows quantised in the kernel)");
+        if (q8 && (batch > 0 || w->wide || w->info.kind == SPTMM_KIND_I2S))
+            return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV is launched alone, on u16 or gap streams");
         if (w->info.kind == SPTMM_KIND_I2S && act != ACT_I8) return fail(SPTMM_ERR_UNSUPPORTED, "the i2s kernel takes int8 activations only");
         const bool batched = batch > 0, lists = w->info.kind != SPTMM_KIND_I2S && !w->wide;
         const int slot = plan_slot(M, batched);
@@ -700,7 +704,7 @@ int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_m
             rc = sptmm_weights_clone(w, &c);
             if (rc == SPTMM_OK) owned.push_back(c), ws.push_back(c);
         }
-        const size_t xbytes = (size_t)M * w->info.K * (act == ACT_I8 ? 1 : act == ACT_F16 ? 2 : 4), cbytes = (size_t)4 * M * w->info.N * per;
+        const size_t xbytes = (size_t)M * w->info.K * (act == ACT_I8 ? 1 : act == ACT_F32 ? 4 : 2), cbytes = (size_t)4 * M * w->info.N * per;
         if (rc == SPTMM_OK) rc = sptmm_malloc(&X, xbytes);
         if (rc == SPTMM_OK) rc = sptmm_malloc(&C, cbytes);
         if (rc == SPTMM_OK) rc = sptmm_memset(X, 0, xbytes);
@@ -718,6 +722,7 @@ int sptmm_weights_tune(sptmm_weights *w, int M, int batch, int act, double *us_m
             for (int p = 0; p < passes; ++p)
                 for (int g = 0; g < groups; ++g) {
                     const int r = batched ? sptmm_gemv_batched(ws.data() + (size_t)g * per, xs.data(), cs.data(), per, M, act, stream)
+                                  : q8    ? gemv_common(ws[g], X, M, C, stream, ACT_I8, 0, nullptr, nullptr, nullptr, act == 3 ? SPTMM_X_F16 : SPTMM_X_BF16, 1.0f)
                                           : gemv_common(ws[g], X, M, C, stream, (ActType)act);
                     if (r != SPTMM_OK) return r;
                 }

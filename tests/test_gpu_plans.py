@@ -114,8 +114,15 @@ def test_fp16_rows_tune_and_refusals(streams):
     Xh = oracle.make_x_normal(5, 4, K, np.float16)
     ref = oracle.sptmm_f64(Xh, pos, neg)
     assert (np.abs(w.matmul(Xh) - ref) / np.maximum(np.abs(ref), np.sqrt(S))).max() <= 1e-3
+    # the quantising GEMV (fp16 rows -> int8 in the kernel) tunes as a lone call; its results stay the float32 arithmetic's
+    us_model, us_tuned, plan = w.tune(4, 0, act=3)
+    say("tune, quantising call:", "model %.3f us -> %.3f us" % (us_model, us_tuned), plan)
+    assert 0 < us_tuned <= us_model
+    q, a = oracle.quantise_rows(Xh.astype(np.float32))
+    assert (w.matmul_q8(Xh, 0.5) == oracle.rescale(oracle.sptmm_i8_mt(q, pos, neg, 8), a, 0.5)).all()
     i2 = makers["i2s"]()
-    for bad in (lambda: i2.tune(1, 0, act=1), lambda: w.tune(0, 0), lambda: w.tune(1, -1), lambda: w.tune(1, 0, act=7), lambda: w.set_plan(0, False)):
+    for bad in (lambda: i2.tune(1, 0, act=1), lambda: w.tune(0, 0), lambda: w.tune(1, -1), lambda: w.tune(1, 0, act=7), lambda: w.set_plan(0, False),
+                lambda: w.tune(4, 8, act=3), lambda: i2.tune(1, 0, act=3)):
         with pytest.raises(sp.SptmmError):
             bad()
     w.free()
