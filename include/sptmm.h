@@ -285,6 +285,15 @@ int sptmm_gemv_f32(const sptmm_weights *w, const float *X_dev, int M, float *C_d
  * an unused scale to its i2s kernel (main.cu:1862).  u16 and gap streams. */
 typedef enum sptmm_xtype { SPTMM_X_F16 = 1, SPTMM_X_BF16 = 2 } sptmm_xtype;
 int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *stream);
+/* The same call with a workspace in device memory (sptmm_gemv_q8_workspace_bytes(w, M) bytes, 256-byte aligned, the
+ * caller's, reusable from call to call on one stream).  With more than four rows, or more than 32 K activation values
+ * in two to four rows, it runs as two launches -- the rows quantised once into the workspace (int8 rows, then their
+ * 1/s), then the int8 GEMV scaling its sums on the way out -- where the fused launch quantises all rows again in every
+ * workgroup (K=6912 N=2560, 8 rows: 19.0 us fused, 11.8 us this way; 16 rows: 35.4 and 13.4); otherwise it is the
+ * fused launch and leaves the workspace alone.  Same arithmetic, same results bit for bit. */
+size_t sptmm_gemv_q8_workspace_bytes(const sptmm_weights *w, int M);
+int sptmm_gemv_q8_ws(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *workspace_dev,
+                     size_t workspace_bytes, void *stream);
 
 /* `count` independent GEMVs of one shape in ONE launch: C[i] = X[i] . ws[i]
  * (int8 activations; streams of one kind that agree in K, N, S, split_k).  What a

@@ -33,7 +33,7 @@ EXPORTS = [
     "sptmm_pack_delta_rows", "sptmm_pack_ragged_rows",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
-    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_i8_batched", "sptmm_gemv_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
+    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_q8_ws", "sptmm_gemv_q8_workspace_bytes", "sptmm_gemv_i8_batched", "sptmm_gemv_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
@@ -102,6 +102,9 @@ def lib() -> C.CDLL:
         for n in ("sptmm_gemv_i8", "sptmm_gemv_f16", "sptmm_gemv_f32"):
             getattr(L, n).argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.sptmm_gemv_q8.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p]
+        L.sptmm_gemv_q8_ws.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.sptmm_gemv_q8_workspace_bytes.argtypes = [C.c_void_p, C.c_int]
+        L.sptmm_gemv_q8_workspace_bytes.restype = C.c_size_t
         L.sptmm_gemv_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_gemv_i8_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_malloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
@@ -602,21 +605,40 @@ class Weights:
         """x_type 1 = fp16, 2 = bf16 (raw 16-bit patterns); Y = float32."""
         _ck(lib().sptmm_gemv_q8(self.handle, X.ptr, x_type, M, w_scale, Yout.ptr, stream.handle if stream else None))
 
-    def matmul_q8(self, X: np.ndarray, w_scale: float = 1.0, bf16: bool = False) -> np.ndarray:
-        """Host convenience: X [M][K] float16 (or uint16 bf16 patterns with bf16=True) -> Y [M][N] float32."""
+    def q8_workspace_bytes(self, M: int) -> int:
+        return int(lib().sptmm_gemv_q8_workspace_bytes(self.handle, M))
+
+    def gemv_q8_ws(self, X: DeviceBuffer, x_type: int, M: int, w_scale: float, Yout: DeviceBuffer, workspace: DeviceBuffer | None,
+                   workspace_bytes: int, stream: Stream | None = None):
+        """gemv_q8 with a device workspace of q8_workspace_bytes(M): beyond four rows, quantise once, then the int8 GEMV."""
+        _ck(lib().sptmm_gemv_q8_ws(self.handle, X.ptr, x_type, M, w_scale, Yout.ptr, workspace.ptr if workspace else None,
+                                   workspace_bytes, stream.handle if stream else None))
+
+    def matmul_q8(self, X: np.ndarray, w_scale: float = 1.0, bf16: bool = False, workspace: bool = False) -> np.ndarray:
+        """Host convenience: X [M][K] float16 (or uint16 bf16 patterns with bf16=True) -> Y [M][N] float32.
+        workspace=True: through gemv_q8_ws with a workspace allocated for the call."""
         i = self.info
         M, K = X.shape
         assert K == i["K"] and X.dtype == (np.uint16 if bf16 else np.float16)
         xb = DeviceBuffer.from_numpy(X)
         yb = DeviceBuffer(4 * M * i["N"])
         yb.fill(0xFF)
+        ws = None
         try:
-            self.gemv_q8(xb, 2 if bf16 else 1, M, w_scale, yb)
+            if workspace:
+                nbytes = self.q8_workspace_bytes(M)
+                ws = DeviceBuffer(nbytes)
+                ws.fill(0xA5)
+                self.gemv_q8_ws(xb, 2 if bf16 else 1, M, w_scale, yb, ws, nbytes)
+            else:
+                self.gemv_q8(xb, 2 if bf16 else 1, M, w_scale, yb)
             device_sync()
             return yb.to_numpy(np.float32, (M, i["N"]))
         finally:
             xb.free()
             yb.free()
+            if ws is not None:
+                ws.free()
 
     def matmul(self, X: np.ndarray) -> np.ndarray:
         """Host convenience: upload X [M][K], run on the device, download C [M][N]."""

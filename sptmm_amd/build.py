@@ -29,7 +29,7 @@ def _run(cmd):
 
 SOURCES = ("formats.cpp", "ragged.cpp", "wide.cpp", "lists_wide.hip", "capi.hip", "i2s.hip", "lists_u16_scaled.hip", "lists_u16_plain.hip",
            "lists_runs8.hip", "lists_runs16.hip", "lists_ragged_u16_scaled.hip", "lists_ragged_u16_plain.hip",
-           "lists_ragged_runs8.hip", "lists_ragged_runs16.hip")
+           "lists_ragged_runs8.hip", "lists_ragged_runs16.hip", "quantise.hip")
 
 
 def build_lib() -> str:

@@ -178,7 +178,7 @@ void fill_args(const sptmm_weights *w, const void *X, int M, void *C, GemvArgs *
 
 int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *stream, ActType act, int batch = 0,
                 const void *const *bw = nullptr, const void *const *bx = nullptr, void *const *bc = nullptr, int quant = 0,
-                float w_scale = 1.f)
+                float w_scale = 1.f, const float *inv = nullptr)
 {
     if (!w || !X || !C) return fail(SPTMM_ERR_INVALID, "null pointer");
     if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
@@ -198,12 +198,13 @@ int gemv_common(const sptmm_weights *w, const void *X, int M, void *C, void *str
     }
     a.quant = quant;
     a.w_scale = w_scale;
+    a.inv = inv;
     a.batch = batch;
     a.batch_w = bw;
     a.batch_X = bx;
     a.batch_C = bc;
     if (w->wide) {
-        if (quant) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
+        if (quant || inv) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
         return launch_wide(a, w->wh, act, stream);
     }
     switch (w->info.kind) {
@@ -846,6 +847,38 @@ int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X, int x_type, int M, 
     if (x_type != SPTMM_X_F16 && x_type != SPTMM_X_BF16) return fail(SPTMM_ERR_INVALID, "x_type must be SPTMM_X_F16 or SPTMM_X_BF16");
     if (w && w->info.kind == SPTMM_KIND_I2S) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes u16 or gap streams");
     return gemv_common(w, X, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, x_type, w_scale);
+}
+
+static bool q8_fused(int M, int K) { return M == 1 || (M <= 4 && (long)M * K <= 32768); }
+// workspace of sptmm_gemv_q8_ws: the int8 rows, then (256-byte aligned) the rows' 1/s
+static size_t q8_rows_bytes(int M, int K) { return ((size_t)M * K + 255) / 256 * 256; }
+
+size_t sptmm_gemv_q8_workspace_bytes(const sptmm_weights *w, int M)
+{
+    if (!w || M < 1) return 0;
+    return q8_rows_bytes(M, w->info.K) + ((size_t)M * sizeof(float) + 255) / 256 * 256;
+}
+
+int sptmm_gemv_q8_ws(const sptmm_weights *w, const uint16_t *X, int x_type, int M, float w_scale, float *Y, void *workspace, size_t workspace_bytes,
+                     void *stream)
+{
+    if (x_type != SPTMM_X_F16 && x_type != SPTMM_X_BF16) return fail(SPTMM_ERR_INVALID, "x_type must be SPTMM_X_F16 or SPTMM_X_BF16");
+    if (!w || !X || !Y) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    if (w->info.kind == SPTMM_KIND_I2S || w->wide) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
+    // The fused launch quantises all the rows again in every workgroup, each reading M x K values twice: up to 32 K values
+    // that is the faster way (K=6912, 4 rows: 8.8 us against 6.2 + 3 in two launches), beyond them it is not (K=6912, 8 rows:
+    // 19.0 against 11.8 us; K=13824, 4 rows: 30.7 us fused).  One row always goes the fused way.
+    if (q8_fused(M, w->info.K)) return gemv_common(w, X, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, x_type, w_scale);
+    const size_t need = sptmm_gemv_q8_workspace_bytes(w, M);
+    if (!workspace || workspace_bytes < need)
+        return fail(SPTMM_ERR_INVALID, "workspace of %zu bytes, %zu needed (sptmm_gemv_q8_workspace_bytes)", workspace ? workspace_bytes : (size_t)0, need);
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
+    float *inv = reinterpret_cast<float *>((uint8_t *)workspace + q8_rows_bytes(M, w->info.K));
+    if (int rc = launch_quantise_rows(X, x_type, M, w->info.K, workspace, inv, stream)) return rc;
+    return gemv_common(w, workspace, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, 0, w_scale, inv);
 }
 
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X, int M, float *C, void *stream)

@@ -193,6 +193,7 @@ struct GemvArgs {
     int stones = 0;       // 8-bit gap stream of tile positions with zero slots behind every 96 rows (RAGGED_MAGIC_STONES)
     int quant = 0;        // 1 / 2: X holds fp16 / bf16 rows, quantised to int8 in the kernel; C receives floats
     float w_scale = 1.f;  // quantising launches: factor applied to every output
+    const float *inv = nullptr;  // int8 rows quantised by an earlier launch: the rows' 1/s on the device; C receives floats (lone list launches, M > 4)
     // batched launch (u16 / gap streams, int8): `batch` GEMVs of this shape, one (w, X, C) triple each
     int batch = 0;
     const void *const *batch_w = nullptr;
@@ -215,6 +216,7 @@ int launch_ragged_runs16(const GemvArgs &a, ActType act, void *stream);      // 
 int launch_delta(const GemvArgs &a, ActType act, void *stream);
 int launch_wide(const GemvArgs &a, const WideHeader &h, ActType act, void *stream);  // lists_wide.hip
 int launch_i2s(const GemvArgs &a, void *stream);
+int launch_quantise_rows(const void *X, int kind, int M, int K, void *Xq, float *inv, void *stream);  // quantise.hip
 int launch_copy(void *dst, const void *src, size_t bytes, void *stream);
 int launch_read(const void *src, size_t bytes, void *sink, int workgroups, void *stream);
 

@@ -510,6 +510,7 @@ struct ListParams {
     // with a vector load whose address waits for a scalar load, two memory round trips in a row before the kernel's
     // first activation or stream load is issued; these arrive with the other arguments in one
     int threads, grid_x;
+    const float *inv;  // kernels for rows quantised beforehand: the rows' 1/s (a / 127), applied to every output
 };
 
 // rows of the activation tile in front of its 64 trailing zero rows
@@ -612,7 +613,9 @@ template <int MT> struct Quantiser {
     }
 };
 
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, bool QUANT = false, bool MERGED = false>
+// QUANT: 0 int8 / float rows as they come; 1 fp16 / bf16 rows quantised to int8 while the tile is staged, floats out;
+// 2 int8 rows quantised beforehand (ListParams::inv holds the rows' 1/s), floats out
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int QUANT = 0, bool MERGED = false>
 struct ListsBody {
     typedef Sums<Act, MT, false, MERGED> SumsT;
     typedef typename Acc<Act>::type A;
@@ -683,7 +686,7 @@ struct ListsBody {
 #pragma unroll
                 for (int m = 0; m < MT; ++m)
                     if (m0 + m < p.M) {
-                        if constexpr (QUANT)
+                        if constexpr (QUANT != 0)
                             Cf[(size_t)(m0 + m) * p.N + col] = (float)v[m] * back[m] * p.w_scale;
                         else
                             C[(size_t)(m0 + m) * p.N + col] = v[m];
@@ -735,9 +738,9 @@ struct ListsBody {
         // 1. every wavefront's activation loads enter the memory pipeline ahead of
         //    any stream load of the workgroup ...
         const int items = p.K / 16;
-        uint4 xr[QUANT ? 1 : St::XI][St::NLOAD];
-        uint4 xq[QUANT && Q::HOLD > 0 ? Q::HOLD : 1][2 * MT];
-        if constexpr (QUANT) {
+        uint4 xr[QUANT == 1 ? 1 : St::XI][St::NLOAD];
+        uint4 xq[QUANT == 1 && Q::HOLD > 0 ? Q::HOLD : 1][2 * MT];
+        if constexpr (QUANT == 1) {
 #pragma unroll
             for (int i = 0; i < Q::HOLD; ++i) {
                 const int item = tid + i * nt;
@@ -776,7 +779,7 @@ struct ListsBody {
         }
 
         // 3. ... and the tile is written while the stream is still in flight.
-        if constexpr (QUANT) {
+        if constexpr (QUANT == 1) {
             // row maxima: own items (held, and beyond them re-read later), wavefront, workgroup
             u32 mb[MT];
 #pragma unroll
@@ -839,7 +842,7 @@ struct ListsBody {
                 for (int i = EARLY; i < RING; ++i) buf[i] = load_round(wp, i < R0 ? i : R0 - 1);
             }
         }
-        if constexpr (!QUANT) {
+        if constexpr (QUANT != 1) {
             for (int item = tid + St::XI * nt; item < items; item += nt) {
                 uint4 r[St::NLOAD];
                 St::load(X, p.M, p.K, m0, item, r);
@@ -881,7 +884,7 @@ struct ListsBody {
         float *Cf = reinterpret_cast<float *>(p.C);  // quantising kernels: acc / s * w_scale
         float back[MT];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) back[m] = QUANT ? qinv[m] : 0.f;
+        for (int m = 0; m < MT; ++m) back[m] = QUANT == 1 ? qinv[m] : QUANT == 2 ? (m0 + m < p.M ? p.inv[m0 + m] : 0.f) : 0.f;
         for (int it = 0; it < p.iters; ++it, task += task_step) {
             const bool active = task < p.tasks;
             const uint8_t *tb = tasks_base + (size_t)(active ? task : 0) * task_bytes;
@@ -1058,8 +1061,8 @@ struct ListsBody {
                         if (p.W == 1) {
                             if (active && lane < (logL == 5 ? 16 : 8) && m0 + m < p.M) {
                                 const int col = (task << (6 - logL)) + (lane >> 3);
-                                if constexpr (QUANT)
-                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)v * qinv[m] * p.w_scale;
+                                if constexpr (QUANT != 0)
+                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)v * (QUANT == 1 ? qinv[m] : p.inv[m0 + m]) * p.w_scale;
                                 else
                                     C[(size_t)(m0 + m) * p.N + col] = v;
                             }
@@ -1097,11 +1100,11 @@ struct ListsBody {
                 if (p.W == 1) {
                     if (active && writer && m0 + m < p.M) {
                         const int cbase = task << (6 - logL);
-                        const float bk = QUANT ? qinv[m] : 0.f;
+                        const float bk = QUANT == 1 ? qinv[m] : QUANT == 2 ? p.inv[m0 + m] : 0.f;
 #pragma unroll
                         for (int x = 0; x < ND; ++x) {
                             if (x > 0 && logL >= 6) break;  // one column per task: tile 1 is already in t[0]
-                            if constexpr (QUANT)
+                            if constexpr (QUANT != 0)
                                 Cf[(size_t)(m0 + m) * p.N + cbase + col[x]] = (float)t[x] * bk * p.w_scale;
                             else
                                 C[(size_t)(m0 + m) * p.N + cbase + col[x]] = t[x];
@@ -1138,7 +1141,7 @@ struct ListsBody {
                         A s = (A)0;
                         for (int w = 0; w < p.W; ++w) s += part[(wave + w) * MT + m];
                         if (m0 + m < p.M) {
-                            if constexpr (QUANT)
+                            if constexpr (QUANT != 0)
                                 Cf[(size_t)(m0 + m) * p.N + col] = (float)s * back[m] * p.w_scale;
                             else
                                 C[(size_t)(m0 + m) * p.N + col] = s;
@@ -1157,8 +1160,8 @@ struct ListsBody {
 // wavefronts then walk tasks blockIdx.x*waves + wave, + gridDim.x*waves, ...
 // blockIdx.y selects the tile of MT activation rows.  RF > 0: every task has
 // exactly RF full rounds (straight-line body); RF == 0: any length (ring).
-template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, bool QUANT = false, bool MERGED = false>
-__global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, QUANT>())) lists_kernel(ListParams p)
+template <typename Act, int MT, int MODE, bool PRE, bool VAR, int RF, int QUANT = 0, bool MERGED = false>
+__global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, QUANT == 1>())) lists_kernel(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     ListsBody<Act, MT, MODE, PRE, VAR, QUANT, MERGED>::template run<RF>(p, smem);
@@ -1169,7 +1172,7 @@ template <bool PRE, int RF, int SL>
 __global__ void __launch_bounds__(1024) lists_kernel_shared(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    ListsBody<int8_t, 1, 0, PRE, false, false, false>::template run<RF, SL>(p, smem);
+    ListsBody<int8_t, 1, 0, PRE, false, 0, false>::template run<RF, SL>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -1188,7 +1191,7 @@ __global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, false>())) list
     p.w = b.w[blockIdx.z];
     p.X = b.X[blockIdx.z];
     p.C = b.C[blockIdx.z];
-    ListsBody<Act, MT, MODE, PRE, VAR, false, MERGED>::template run<RF>(p, smem);
+    ListsBody<Act, MT, MODE, PRE, VAR, 0, MERGED>::template run<RF>(p, smem);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -1230,7 +1233,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
     int regs = vgprs.load(std::memory_order_relaxed);
     if (!regs) {
         hipFuncAttributes fa;
-        hipError_t e = hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(lists_kernel<Act, MT, MODE, PRE, VAR, RF, false, MERGED>));
+        hipError_t e = hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(lists_kernel<Act, MT, MODE, PRE, VAR, RF, 0, MERGED>));
         if (e != hipSuccess) return hip_fail(e, "hipFuncGetAttributes");
         regs = fa.numRegs > 0 ? fa.numRegs : 128;
         vgprs.store(regs, std::memory_order_relaxed);
@@ -1408,9 +1411,23 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             return SPTMM_OK;
         }
     }
+    if (a.inv) {
+        // rows quantised by an earlier launch (sptmm_gemv_q8_ws): the int8 kernel, its sums scaled on the way out
+        if constexpr (MT >= 4 && sizeof(Act) == 1 && !is_byte_rows<Act>()) {
+            auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, 2, MERGED>;
+            p.inv = a.inv;
+            static std::atomic<size_t> lds_granted_p{48 * 1024};
+            if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted_p)) return rc;
+            hipLaunchKernelGGL(kern, grid, block, lds, st, p);
+            hipError_t e = hipGetLastError();
+            return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel (rows quantised beforehand) launch");
+        } else {
+            return fail(SPTMM_ERR_INVALID, "rows quantised beforehand go through the four- and eight-row int8 kernels");
+        }
+    }
     if (a.quant) {
         if constexpr (sizeof(Act) == 1 && !is_byte_rows<Act>()) {  // (quantising launches never take the byte tile: no such kernels are built)
-            auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, true, MERGED>;
+            auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, 1, MERGED>;
             // + room for the per-wavefront sums of a full workgroup, the row maxima and the rows' 1/s
             lds = tile + (size_t)(2 * LISTS_MAX_WAVES + 1) * MT * 4;
             if ((int)lds > a.lds_limit) return fail(SPTMM_ERR_UNSUPPORTED, "activation tile of %zu bytes exceeds the LDS limit %d", lds, a.lds_limit);
@@ -1423,7 +1440,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             return fail(SPTMM_ERR_INVALID, "quantising launches go through the int8 kernels");
         }
     }
-    auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, false, MERGED>;
+    auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, 0, MERGED>;
     static std::atomic<size_t> lds_granted{48 * 1024};
     if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
     hipLaunchKernelGGL(kern, grid, block, lds, st, p);

@@ -110,3 +110,87 @@ def test_q8_argument_errors():
         o.free()
     xb.free()
     yb.free()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_q8_with_a_workspace_is_the_same_arithmetic(dtype):
+    """sptmm_gemv_q8_ws: beyond four rows the rows are quantised once by a launch of their own and the int8 GEMV scales its
+    sums on the way out; up to four rows it is the fused launch.  Either way the floats are the fused call's, bit for bit,
+    and the float32 arithmetic's around the oracle's integer sums -- balanced and ragged streams, every lanes-per-column
+    case of the eight-row tiles, row counts that leave the last tile partly filled."""
+    K, N, S = 2560, 640, 1536
+    Wd, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    ragged = sp.generate_ternary_iid(K, N, 0x99, 0.25, 0.35)
+    streams = [("u16 %d" % sk, sp.Weights.upload_u16(pos, neg, K, sk), None) for sk in (8, 16, 32, 64, 128)]
+    streams += [("gap %d" % sk, sp.Weights.upload_delta(pos, neg, K, sk), None) for sk in (8, 32, 64)]
+    streams += [("gap for one row", sp.Weights.upload_delta(pos, neg, K, 32, rows=1), None)]
+    streams += [("ragged u16", sp.Weights.upload_dense(ragged, sp.KIND_U16, 32), ragged), ("ragged gap", sp.Weights.upload_dense(ragged, sp.KIND_DELTA, 16), ragged)]
+    try:
+        for name, w, dense in streams:
+            for M in (1, 4, 5, 8, 9, 13, 16, 20):
+                print("q8 workspace", name, dtype, "M", M, flush=True)
+                sys.stdout.flush()
+                X, xf = rows(300 + M, M, K, dtype)
+                if M >= 9:
+                    xf[M - 1] = 0  # a row of zeros: its scale clamps at 1e-5
+                    X[M - 1] = 0
+                q, a = quantise_ref(xf)
+                C = oracle.sptmm_i8_mt(q, pos, neg, 8) if dense is None else oracle.dense_i8(q, dense)
+                want = y_ref(C, a, 0.25)
+                got = w.matmul_q8(X, w_scale=0.25, bf16=dtype == "bf16", workspace=True)
+                assert (got == want).all(), (name, M, np.abs(got - want).max())
+                assert (got == w.matmul_q8(X, w_scale=0.25, bf16=dtype == "bf16")).all(), (name, M)
+    finally:
+        for _, w, _ in streams:
+            w.free()
+
+
+def test_q8_workspace_is_checked_and_reusable():
+    K, N, S = 6912, 2560, 4096
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    w = sp.Weights.upload_u16(pos, neg, K, 32)
+    i2 = sp.Weights.upload_i2s(sp.generate_ternary(256, 32, 64, dense=True)[0])
+    M = 8
+    need = w.q8_workspace_bytes(M)
+    assert need >= M * K + 4 * M and need % 256 == 0 and w.q8_workspace_bytes(16) > need
+    ws = sp.DeviceBuffer(need)
+    yb = sp.DeviceBuffer(4 * M * N)
+    st = sp.Stream()
+    try:
+        for seed in (1, 2, 3):  # one workspace, call after call on one stream
+            X, xf = rows(seed, M, K, "f16")
+            xb = sp.DeviceBuffer.from_numpy(X)
+            w.gemv_q8_ws(xb, 1, M, 1.0, yb, ws, need, st)
+            st.sync()
+            q, a = quantise_ref(xf)
+            assert (yb.to_numpy(np.float32, (M, N)) == y_ref(oracle.sptmm_i8_mt(q, pos, neg, 8), a, 1.0)).all()
+            xb.free()
+        X, _ = rows(9, M, K, "f16")
+        xb = sp.DeviceBuffer.from_numpy(X)
+        for bad in (lambda: w.gemv_q8_ws(xb, 1, M, 1.0, yb, ws, need - 1, st), lambda: w.gemv_q8_ws(xb, 1, M, 1.0, yb, None, need, st),
+                    lambda: w.gemv_q8_ws(xb, 3, M, 1.0, yb, ws, need, st), lambda: i2.gemv_q8_ws(xb, 1, M, 1.0, yb, ws, need, st)):
+            with pytest.raises(sp.SptmmError):
+                bad()
+        w.gemv_q8_ws(xb, 1, 4, 1.0, yb, None, 0, st)  # up to four rows: the fused launch, no workspace needed
+        st.sync()
+        xb.free()
+    finally:
+        for o in (ws, yb, w, i2):
+            o.free()
+
+
+def test_q8_workspace_with_few_rows_of_a_long_k():
+    """Two to four rows of more than 32 K values go the two-launch way as well (four-row int8 tiles scaling their sums on
+    the way out); one row never does."""
+    K, N, S = 13824, 1280, 8320
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    for name, w in (("u16", sp.Weights.upload_u16(pos, neg, K, 0)), ("gap", sp.Weights.upload_delta(pos, neg, K, 0)), ("u16 64", sp.Weights.upload_u16(pos, neg, K, 64))):
+        for M in (1, 2, 3, 4):
+            print("q8 workspace, long K", name, "M", M, flush=True)
+            sys.stdout.flush()
+            X, xf = rows(500 + M, M, K, "f16")
+            q, a = quantise_ref(xf)
+            want = y_ref(oracle.sptmm_i8_mt(q, pos, neg, 8), a, 2.0)
+            assert (w.matmul_q8(X, w_scale=2.0, workspace=True) == want).all(), (name, M)
+            assert (w.matmul_q8(X, w_scale=2.0) == want).all(), (name, M)
+        w.free()
