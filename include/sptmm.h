@@ -294,6 +294,16 @@ int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int
 size_t sptmm_gemv_q8_workspace_bytes(const sptmm_weights *w, int M);
 int sptmm_gemv_q8_ws(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *workspace_dev,
                      size_t workspace_bytes, void *stream);
+/* sptmm_gemv_q8_ws without a workspace of the caller's and without any allocation, for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * The workspace is a static array in the library's device image (528,384 bytes on every GPU the library runs on, until
+ * the process ends; its address is looked up per device in sptmm_device_init, or at the first call on a device):
+ * calls whose workspace would be larger (sptmm_gemv_q8_workspace_bytes: M x K int8 values and M floats, each rounded
+ * up to 256 bytes -- 38 rows at K = 13824 still fit) return SPTMM_ERR_UNSUPPORTED.  All calls on one GPU share the one array:
+ * calls that overlap on a GPU (different streams, or threads) race on it -- serialise them, or use sptmm_gemv_q8_ws.
+ * Nothing in it has to start at zero (every call rewrites the rows and scales it reads).  Same floats as
+ * sptmm_gemv_q8_ws and sptmm_gemv_q8, bit for bit. */
+int sptmm_gemv_q8_static(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *stream);
 
 /* `count` independent GEMVs of one shape in ONE launch: C[i] = X[i] . ws[i]
  * (int8 activations; streams of one kind that agree in K, N, S, split_k).  What a

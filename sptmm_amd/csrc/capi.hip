@@ -230,6 +230,7 @@ int sptmm_device_init(int device, sptmm_devinfo *out)
         if (device < 0 || device >= count) return fail(SPTMM_ERR_INVALID, "device %d out of range (have %d)", device, count);
         HIP_TRY(hipSetDevice(device));
         tuning_reload();  // the launch-shape overrides of tuning runs: read here, never on a launch path
+        if (int rc = scratch_init(device)) return rc;  // this device's copy of the static scratch (sptmm_gemv_q8_static)
         if (out) {
             hipDeviceProp_t pr;
             HIP_TRY(hipGetDeviceProperties(&pr, device));
@@ -853,6 +854,14 @@ static bool q8_fused(int M, int K) { return M == 1 || (M <= 4 && (long)M * K <= 
 // workspace of sptmm_gemv_q8_ws: the int8 rows, then (256-byte aligned) the rows' 1/s
 static size_t q8_rows_bytes(int M, int K) { return ((size_t)M * K + 255) / 256 * 256; }
 
+// the rows quantised into `workspace` (int8 rows, then their 1/s), then the int8 GEMV scaling its sums by them
+static int q8_two_launches(const sptmm_weights *w, const uint16_t *X, int x_type, int M, float w_scale, float *Y, void *workspace, void *stream)
+{
+    float *inv = reinterpret_cast<float *>((uint8_t *)workspace + q8_rows_bytes(M, w->info.K));
+    if (int rc = launch_quantise_rows(X, x_type, M, w->info.K, workspace, inv, stream)) return rc;
+    return gemv_common(w, workspace, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, 0, w_scale, inv);
+}
+
 size_t sptmm_gemv_q8_workspace_bytes(const sptmm_weights *w, int M)
 {
     if (!w || M < 1) return 0;
@@ -876,9 +885,26 @@ int sptmm_gemv_q8_ws(const sptmm_weights *w, const uint16_t *X, int x_type, int 
     int dev = -1;
     HIP_TRY(hipGetDevice(&dev));
     if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
-    float *inv = reinterpret_cast<float *>((uint8_t *)workspace + q8_rows_bytes(M, w->info.K));
-    if (int rc = launch_quantise_rows(X, x_type, M, w->info.K, workspace, inv, stream)) return rc;
-    return gemv_common(w, workspace, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, 0, w_scale, inv);
+    return q8_two_launches(w, X, x_type, M, w_scale, Y, workspace, stream);
+}
+
+int sptmm_gemv_q8_static(const sptmm_weights *w, const uint16_t *X, int x_type, int M, float w_scale, float *Y, void *stream)
+{
+    if (x_type != SPTMM_X_F16 && x_type != SPTMM_X_BF16) return fail(SPTMM_ERR_INVALID, "x_type must be SPTMM_X_F16 or SPTMM_X_BF16");
+    if (!w || !X || !Y) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (M < 1) return fail(SPTMM_ERR_INVALID, "M must be at least 1");
+    if (w->info.kind == SPTMM_KIND_I2S || w->wide) return fail(SPTMM_ERR_UNSUPPORTED, "the quantising GEMV takes the ordinary u16 or gap streams");
+    if (q8_fused(M, w->info.K)) return gemv_common(w, X, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, x_type, w_scale);  // (no scratch in that launch)
+    const size_t need = sptmm_gemv_q8_workspace_bytes(w, M);
+    if (need > scratch_bytes())
+        return fail(SPTMM_ERR_UNSUPPORTED, "%d rows of K = %d need %zu bytes of scratch, the static array holds %zu: use sptmm_gemv_q8_ws", M, w->info.K,
+                    need, scratch_bytes());
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev != w->device) return fail(SPTMM_ERR_INVALID, "the weights live on device %d but device %d is current", w->device, dev);
+    void *ptr = nullptr;
+    if (int rc = scratch_of(dev, &ptr)) return rc;
+    return q8_two_launches(w, X, x_type, M, w_scale, Y, ptr, stream);
 }
 
 int sptmm_gemv_f16(const sptmm_weights *w, const uint16_t *X, int M, float *C, void *stream)

@@ -217,6 +217,9 @@ int launch_delta(const GemvArgs &a, ActType act, void *stream);
 int launch_wide(const GemvArgs &a, const WideHeader &h, ActType act, void *stream);  // lists_wide.hip
 int launch_i2s(const GemvArgs &a, void *stream);
 int launch_quantise_rows(const void *X, int kind, int M, int K, void *Xq, float *inv, void *stream);  // quantise.hip
+size_t scratch_bytes();                     // the library's static device scratch (quantise.hip): its size,
+int scratch_init(int device);               // the look-up of its address on the current device (sptmm_device_init),
+int scratch_of(int device, void **ptr);     // and that address
 int launch_copy(void *dst, const void *src, size_t bytes, void *stream);
 int launch_read(const void *src, size_t bytes, void *sink, int workgroups, void *stream);
 

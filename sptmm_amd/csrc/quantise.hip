@@ -49,4 +49,39 @@ int launch_quantise_rows(const void *X, int kind, int M, int K, void *Xq, float 
     return e == hipSuccess ? SPTMM_OK : fail(SPTMM_ERR_HIP, "quantise_rows_kernel launch: %s (%d)", hipGetErrorString(e), (int)e);
 }
 
+// ---- scratch for callers that cannot allocate (sptmm_gemv_q8_static): the workspace of sptmm_gemv_q8_ws, in the library's
+// own device image.  Every GPU the library runs on holds its copy of the array until the process ends, each at its own
+// address; `scratch` is only the host-side name of the symbol -- what kernels and copies take is the device address
+// looked up below, once per device.
+constexpr size_t SCRATCH_BYTES = 512 * 1024 + 4096;  // the int8 activation values (M x K, some 524,000 of them at most), then the rows' 1/s
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[SCRATCH_BYTES];  // (no kernel names it: kept for the look-up)
+constexpr int SCRATCH_DEVICES = 64;
+static std::atomic<void *> scratch_ptr[SCRATCH_DEVICES];
+
+size_t scratch_bytes() { return SCRATCH_BYTES; }
+
+// with `device` current: look up and keep the address of this device's copy of the array
+int scratch_init(int device)
+{
+    if (device < 0 || device >= SCRATCH_DEVICES) return SPTMM_OK;  // (no slot to keep it in: scratch_of says so when asked)
+    void *ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return fail(SPTMM_ERR_HIP, "hipGetSymbolAddress(scratch): %s (%d)", hipGetErrorString(e), (int)e);
+    scratch_ptr[device].store(ptr, std::memory_order_release);
+    return SPTMM_OK;
+}
+
+// the device address of `device`'s copy (looked up now if sptmm_device_init has not run for it; `device` must be current)
+int scratch_of(int device, void **ptr)
+{
+    if (device < 0 || device >= SCRATCH_DEVICES) return fail(SPTMM_ERR_UNSUPPORTED, "static scratch is kept for devices 0..%d", SCRATCH_DEVICES - 1);
+    void *p = scratch_ptr[device].load(std::memory_order_acquire);
+    if (!p) {
+        if (int rc = scratch_init(device)) return rc;
+        p = scratch_ptr[device].load(std::memory_order_acquire);
+    }
+    *ptr = p;
+    return SPTMM_OK;
+}
+
 }  // namespace sptmm
