@@ -68,3 +68,36 @@ def test_static_scratch_refuses_what_does_not_fit():
     finally:
         for o in (xb, yb, w):
             o.free()
+
+
+def test_static_scratch_call_under_graph_capture():
+    """The caller this entry point is for: a captured stream, where nothing may be allocated.  Three replays with new
+    activations in the captured buffer, eager work between them, each against the workspace call's floats."""
+    sp.device_init(0)
+    K, N, S, M = 6912, 2560, 4096, 8
+    _, pos, neg = sp.generate_ternary(K, N, S)
+    w = sp.Weights.upload_delta(pos, neg, K, 0)
+    st = sp.Stream()
+    xb = sp.DeviceBuffer(2 * M * K)
+    need = w.q8_workspace_bytes(M)
+    ws, y_graph, y_eager = sp.DeviceBuffer(need), sp.DeviceBuffer(4 * M * N), sp.DeviceBuffer(4 * M * N)
+    try:
+        xb.upload(sp.make_x_normal(1, M, K))
+        with sp.Graph(st) as g:
+            w.gemv_q8_static(xb, 1, M, 0.125, y_graph, st)
+        st.sync()
+        for rep in range(3):
+            say("no-alloc q8 under capture: replay", rep)
+            xb.upload(sp.make_x_normal(100 + rep, M, K))
+            y_graph.fill(0xFF)
+            y_eager.fill(0xEE)
+            g.launch(st)
+            st.sync()
+            w.gemv_q8_ws(xb, 1, M, 0.125, y_eager, ws, need, st)  # eager work between the replays
+            st.sync()
+            a, b = y_graph.to_numpy(np.uint32, (M, N)), y_eager.to_numpy(np.uint32, (M, N))
+            assert (a == b).all() and (a != 0xFFFFFFFF).all(), rep
+        g.destroy()
+    finally:
+        for o in (xb, ws, y_graph, y_eager, w):
+            o.free()
