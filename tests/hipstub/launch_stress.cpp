@@ -56,6 +56,19 @@ static void hammer(int K, int N, int S, int split, int launches)
             OK(sptmm_measure_gemv(ws.data(), 8, 2, x, 4, c, launches / 4, 0, st, &us));
             OK(sptmm_measure_gemv(ws.data(), 8, 3, x, 4, c, launches / 4, 0, st, &us));
         }
+        if (w == u || w == d || w == rag) {
+            // the quantising GEMV: fused, with a workspace of the caller's, on the library's static device array
+            void *ws = nullptr;
+            const size_t ws_bytes = sptmm_gemv_q8_workspace_bytes(w, 16);
+            OK(sptmm_malloc(&ws, ws_bytes));
+            for (int i = 0; i < launches / 8; ++i) {
+                const int m = 1 + i % 16;
+                OK(sptmm_gemv_q8(w, (const uint16_t *)x, SPTMM_X_F16, m, 0.5f, (float *)c, st));
+                OK(sptmm_gemv_q8_ws(w, (const uint16_t *)x, SPTMM_X_BF16, m, 0.5f, (float *)c, ws, ws_bytes, st));
+                OK(sptmm_gemv_q8_static(w, (const uint16_t *)x, SPTMM_X_F16, m, 0.5f, (float *)c, st));
+            }
+            OK(sptmm_free(ws));
+        }
         std::vector<sptmm_step> steps;
         for (int i = 0; i < 28; ++i) steps.push_back(sptmm_step{ws[i], x, c, 1 + i % 4 * 5, 0, i / 3});
         for (int mode = 0; mode <= 4; ++mode) OK(sptmm_measure_sequence(steps.data(), (int)steps.size(), launches / 28, mode, st, &us));
