@@ -285,7 +285,11 @@ int sptmm_gemv_f32(const sptmm_weights *w, const float *X_dev, int M, float *C_d
  * an unused scale to its i2s kernel (main.cu:1862).  u16 and gap streams. */
 typedef enum sptmm_xtype { SPTMM_X_F16 = 1, SPTMM_X_BF16 = 2 } sptmm_xtype;
 int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X_dev, int x_type, int M, float w_scale, float *Y_dev, void *stream);
-/* The same call with a workspace in device memory (sptmm_gemv_q8_workspace_bytes(w, M) bytes, 256-byte aligned, the
+/* The rescale alone, for callers whose activations are int8 already (quantised by the operator in front, which also
+ * left the rows' 1/s_m -- a_m / 127 -- in device memory): the sums of sptmm_gemv_i8 written as
+ * Y[m][n] = (float)C[m][n] * inv_scale[m] * w_scale, in this order, by the GEMV's own launch.  u16 and gap streams. */
+int sptmm_gemv_i8_scaled(const sptmm_weights *w, const int8_t *Xq_dev, const float *inv_scale_dev, int M, float w_scale, float *Y_dev, void *stream);
+/* sptmm_gemv_q8 with a workspace in device memory (sptmm_gemv_q8_workspace_bytes(w, M) bytes, 256-byte aligned, the
  * caller's, reusable from call to call on one stream).  With more than four rows, or more than 32 K activation values
  * in two to four rows, it runs as two launches -- the rows quantised once into the workspace (int8 rows, then their
  * 1/s), then the int8 GEMV scaling its sums on the way out -- where the fused launch quantises all rows again in every

@@ -33,7 +33,7 @@ EXPORTS = [
     "sptmm_pack_delta_rows", "sptmm_pack_ragged_rows",
     "sptmm_weights_upload_i2s", "sptmm_weights_clone", "sptmm_weights_save", "sptmm_weights_load",
     "sptmm_weights_free", "sptmm_weights_info", "sptmm_weights_bytes", "sptmm_gemv_i8", "sptmm_gemv_f16",
-    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_q8_ws", "sptmm_gemv_q8_workspace_bytes", "sptmm_gemv_q8_static", "sptmm_gemv_i8_batched", "sptmm_gemv_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
+    "sptmm_gemv_f32", "sptmm_gemv_q8", "sptmm_gemv_q8_ws", "sptmm_gemv_q8_workspace_bytes", "sptmm_gemv_q8_static", "sptmm_gemv_i8_scaled", "sptmm_gemv_i8_batched", "sptmm_gemv_batched", "sptmm_malloc", "sptmm_free", "sptmm_memcpy_h2d", "sptmm_memcpy_d2h", "sptmm_memset",
     "sptmm_stream_create", "sptmm_stream_destroy", "sptmm_stream_sync", "sptmm_device_sync",
     "sptmm_event_create", "sptmm_event_destroy", "sptmm_event_record", "sptmm_event_sync",
     "sptmm_event_elapsed_us", "sptmm_measure_gemv", "sptmm_copy_kernel", "sptmm_read_kernel",
@@ -105,6 +105,7 @@ def lib() -> C.CDLL:
         L.sptmm_gemv_q8_ws.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         L.sptmm_gemv_q8_workspace_bytes.argtypes = [C.c_void_p, C.c_int]
         L.sptmm_gemv_q8_static.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p]
+        L.sptmm_gemv_i8_scaled.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_void_p]
         L.sptmm_gemv_q8_workspace_bytes.restype = C.c_size_t
         L.sptmm_gemv_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.sptmm_gemv_i8_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
@@ -614,6 +615,24 @@ class Weights:
         """gemv_q8 with a device workspace of q8_workspace_bytes(M): beyond four rows, quantise once, then the int8 GEMV."""
         _ck(lib().sptmm_gemv_q8_ws(self.handle, X.ptr, x_type, M, w_scale, Yout.ptr, workspace.ptr if workspace else None,
                                    workspace_bytes, stream.handle if stream else None))
+
+    def gemv_i8_scaled(self, Xq: DeviceBuffer, inv: DeviceBuffer, M: int, w_scale: float, Yout: DeviceBuffer, stream: Stream | None = None):
+        """int8 rows quantised beforehand + their 1/s (float32 [M]) -> Y = float32(C) * inv[m] * w_scale."""
+        _ck(lib().sptmm_gemv_i8_scaled(self.handle, Xq.ptr, inv.ptr, M, w_scale, Yout.ptr, stream.handle if stream else None))
+
+    def matmul_i8_scaled(self, Xq: np.ndarray, inv: np.ndarray, w_scale: float = 1.0) -> np.ndarray:
+        i = self.info
+        M, K = Xq.shape
+        assert K == i["K"] and Xq.dtype == np.int8 and inv.dtype == np.float32 and inv.shape == (M,)
+        xb, ib, yb = DeviceBuffer.from_numpy(Xq), DeviceBuffer.from_numpy(inv), DeviceBuffer(4 * M * i["N"])
+        yb.fill(0xFF)
+        try:
+            self.gemv_i8_scaled(xb, ib, M, w_scale, yb)
+            device_sync()
+            return yb.to_numpy(np.float32, (M, i["N"]))
+        finally:
+            for o in (xb, ib, yb):
+                o.free()
 
     def gemv_q8_static(self, X: DeviceBuffer, x_type: int, M: int, w_scale: float, Yout: DeviceBuffer, stream: Stream | None = None):
         """gemv_q8_ws on the library's static device scratch: allocates nothing; calls that overlap on one GPU race."""

@@ -850,6 +850,13 @@ int sptmm_gemv_q8(const sptmm_weights *w, const uint16_t *X, int x_type, int M, 
     return gemv_common(w, X, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, x_type, w_scale);
 }
 
+int sptmm_gemv_i8_scaled(const sptmm_weights *w, const int8_t *Xq, const float *inv, int M, float w_scale, float *Y, void *stream)
+{
+    if (!inv) return fail(SPTMM_ERR_INVALID, "null pointer");
+    if (w && (w->info.kind == SPTMM_KIND_I2S || w->wide)) return fail(SPTMM_ERR_UNSUPPORTED, "scaled sums come from the ordinary u16 or gap streams");
+    return gemv_common(w, Xq, M, Y, stream, ACT_I8, 0, nullptr, nullptr, nullptr, 0, w_scale, inv);
+}
+
 static bool q8_fused(int M, int K) { return M == 1 || (M <= 4 && (long)M * K <= 32768); }
 // workspace of sptmm_gemv_q8_ws: the int8 rows, then (256-byte aligned) the rows' 1/s
 static size_t q8_rows_bytes(int M, int K) { return ((size_t)M * K + 255) / 256 * 256; }

@@ -710,7 +710,7 @@ struct ListsBody {
     template <int RF, int SL = 0>
     static __device__ __forceinline__ void run(const ListParams &p, unsigned char *smem)
     {
-        static_assert(SL == 0 || (RF > 0 && MODE == 0 && !VAR && !QUANT && MT == 1 && sizeof(Act) == 1), "shared tasks: u16 lists, one int8 row");
+        static_assert(SL == 0 || (RF > 0 && MODE == 0 && !VAR && QUANT != 1 && MT == 1 && sizeof(Act) == 1), "shared tasks: u16 lists, one int8 row");
         constexpr int NR = RF > 0 ? RF : 0;               // full rounds of the straight-line body (RF == -1: none, tails only)
         constexpr int NB = RF > 0 ? RF : RF == 0 ? RING : 1;
         // stepping-stone streams: item i (16 rows) goes to item i + i/6 of the tile, every seventh item stays zero
@@ -1124,7 +1124,10 @@ struct ListsBody {
                     A sum = (A)0;
 #pragma unroll
                     for (int w = 0; w < (1 << SL); ++w) sum += part[(wave + w) * 8 + lane];
-                    C[(size_t)m0 * p.N + (task << (6 - p.logL)) + lane] = sum;
+                    if constexpr (QUANT != 0)
+                        Cf[(size_t)m0 * p.N + (task << (6 - p.logL)) + lane] = (float)sum * back[0] * p.w_scale;
+                    else
+                        C[(size_t)m0 * p.N + (task << (6 - p.logL)) + lane] = sum;
                 }
                 if (it + 1 < p.iters) __syncthreads();  // (the next task's sums go to the same place)
             } else {
@@ -1168,11 +1171,11 @@ __global__ void __launch_bounds__((64 * lists_max_waves<Act, MT, QUANT == 1>()))
 }
 
 // One int8 row on u16 lists with 1 << SL wavefronts per task (see ListsBody::run): up to 16 wavefronts per workgroup.
-template <bool PRE, int RF, int SL>
+template <bool PRE, int RF, int SL, int QUANT = 0>
 __global__ void __launch_bounds__(1024) lists_kernel_shared(ListParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    ListsBody<int8_t, 1, 0, PRE, false, 0, false>::template run<RF, SL>(p, smem);
+    ListsBody<int8_t, 1, 0, PRE, false, QUANT, false>::template run<RF, SL>(p, smem);
 }
 
 // Several independent GEMVs of one shape in one launch: blockIdx.z picks the
@@ -1412,8 +1415,8 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
         }
     }
     if (a.inv) {
-        // rows quantised by an earlier launch (sptmm_gemv_q8_ws): the int8 kernel, its sums scaled on the way out
-        if constexpr (MT >= 4 && sizeof(Act) == 1 && !is_byte_rows<Act>()) {
+        // rows quantised beforehand (sptmm_gemv_i8_scaled, sptmm_gemv_q8_ws): the int8 kernel, its sums scaled on the way out
+        if constexpr (sizeof(Act) == 1) {
             auto kern = lists_kernel<Act, MT, MODE, PRE, VAR, RF, 2, MERGED>;
             p.inv = a.inv;
             static std::atomic<size_t> lds_granted_p{48 * 1024};
@@ -1422,7 +1425,7 @@ static int launch_lists_rf(const GemvArgs &a, hipStream_t st)
             hipError_t e = hipGetLastError();
             return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel (rows quantised beforehand) launch");
         } else {
-            return fail(SPTMM_ERR_INVALID, "rows quantised beforehand go through the four- and eight-row int8 kernels");
+            return fail(SPTMM_ERR_INVALID, "rows quantised beforehand go through the int8 kernels");
         }
     }
     if (a.quant) {
@@ -1462,10 +1465,12 @@ static int launch_lists_shared(const GemvArgs &a, int wpb, hipStream_t st)
     const int grid_x = blocks < slots ? blocks : slots;
     const int iters = (blocks + grid_x - 1) / grid_x;
     ListParams p{(const uint8_t *)a.w, a.X, a.C, a.M, a.K, a.N, a.n_lane, a.tasks, ilog2(a.L), a.W,
-                 0, 0, iters, 0, 1.f, 0, 64 * wpb, grid_x};
-    auto kern = lists_kernel_shared<PRE, RF, SL>;
-    static std::atomic<size_t> lds_granted{48 * 1024};
-    if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, lds_granted)) return rc;
+                 0, 0, iters, 0, a.w_scale, 0, 64 * wpb, grid_x};
+    p.inv = a.inv;
+    // (a row quantised beforehand: the same kernel with its sums scaled on the way out)
+    auto kern = a.inv ? lists_kernel_shared<PRE, RF, SL, 2> : lists_kernel_shared<PRE, RF, SL, 0>;
+    static std::atomic<size_t> lds_granted{48 * 1024}, lds_granted_p{48 * 1024};
+    if (int rc = grant_lds(reinterpret_cast<const void *>(kern), lds, a.inv ? lds_granted_p : lds_granted)) return rc;
     hipLaunchKernelGGL(kern, dim3(grid_x), dim3(64 * wpb), lds, st, p);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? SPTMM_OK : hip_fail(e, "lists_kernel_shared launch");

@@ -194,3 +194,42 @@ def test_q8_workspace_with_few_rows_of_a_long_k():
             assert (w.matmul_q8(X, w_scale=2.0, workspace=True) == want).all(), (name, M)
             assert (w.matmul_q8(X, w_scale=2.0) == want).all(), (name, M)
         w.free()
+
+
+def test_int8_rows_with_their_scales_go_through_one_launch():
+    """sptmm_gemv_i8_scaled: activations quantised by the caller (int8 rows and a / 127 per row) -> the floats of the
+    quantising call, from the int8 GEMV's own launch: every row count class (the lone one-row kernels with two wavefronts
+    per task and on the byte tile included), balanced, ragged and sparse streams, columns that span wavefronts."""
+    K, N, S = 2560, 640, 1536
+    Wd, pos, neg = sp.generate_ternary(K, N, S, dense=True)
+    ragged = sp.generate_ternary_iid(K, N, 0x42, 0.2, 0.3)
+    sparse = sp.generate_ternary_iid(K, N, 0x43, 0.02, 0.03)
+    streams = [("u16 %d" % sk, sp.Weights.upload_u16(pos, neg, K, sk), None) for sk in (8, 16, 32, 64, 128, 256)]
+    streams += [("gap %d" % sk, sp.Weights.upload_delta(pos, neg, K, sk), None) for sk in (16, 64)]
+    streams += [("gap for one row", sp.Weights.upload_delta(pos, neg, K, 32, rows=1), None)]
+    streams += [("ragged u16", sp.Weights.upload_dense(ragged, sp.KIND_U16, 32), ragged), ("ragged gap", sp.Weights.upload_dense(ragged, sp.KIND_DELTA, 16), ragged),
+                ("sparse gap", sp.Weights.upload_dense(sparse, sp.KIND_DELTA, 8), sparse), ("sparse gap for one row", sp.Weights.upload_dense(sparse, sp.KIND_DELTA, 8, rows=1), sparse)]
+    try:
+        for name, w, dense in streams:
+            for M in (1, 2, 4, 5, 8, 11):
+                print("i8 scaled", name, "M", M, flush=True)
+                sys.stdout.flush()
+                _, xf = rows(700 + M, M, K, "f16")
+                q, a = quantise_ref(xf)
+                inv = (a / np.float32(127.0)).astype(np.float32)
+                C = oracle.sptmm_i8_mt(q, pos, neg, 8) if dense is None else oracle.dense_i8(q, dense)
+                got = w.matmul_i8_scaled(q, inv, 0.3)
+                assert got.dtype == np.float32 and (got == y_ref(C, a, 0.3)).all(), (name, M)
+        big = sp.Weights.upload_u16(*sp.generate_ternary(6912, 2560, 4096)[1:], 6912, 32)  # the headline: two wavefronts per task at M = 1
+        _, xf = rows(9, 1, 6912, "f16")
+        q, a = quantise_ref(xf)
+        _, bp, bn = sp.generate_ternary(6912, 2560, 4096)
+        assert (big.matmul_i8_scaled(q, (a / np.float32(127.0)).astype(np.float32), 2.0) == y_ref(oracle.sptmm_i8_mt(q, bp, bn, 8), a, 2.0)).all()
+        big.free()
+        i2 = sp.Weights.upload_i2s(Wd)
+        with pytest.raises(sp.SptmmError):
+            i2.matmul_i8_scaled(q[:, :K] if q.shape[1] >= K else np.zeros((1, K), np.int8), np.ones(1, np.float32))
+        i2.free()
+    finally:
+        for _, w, _ in streams:
+            w.free()
