@@ -189,6 +189,55 @@ def layer_sequence(sp, st, checks, reps):
                         "us per layer between two HIP events around `reps` passes (sptmm_measure_sequence)"}
 
 
+def quantising_leg(sp, st, k_rows, n_cols, s_nz, calls=600):
+    """The calls around the int8 GEMV that BitNet inference makes (not in the reference, which has the GEMV only): one
+    call per launch sequence, HBM-cold (rotating over device copies of the stream), microseconds per call by the host's
+    clock around `calls` calls and a stream synchronise: the int8 GEMV, the same with its sums scaled on the way out
+    (rows quantised by the caller), the fused quantising launch on fp16 rows, and its workspace variant (beyond four
+    rows: the rows quantised once in a launch of their own)."""
+    import numpy as np
+
+    _, p, n = sp.generate_ternary(k_rows, n_cols, s_nz)
+    rows = []
+    for enc in ("u16", "delta"):
+        for m in (1, 4, 8, 16):
+            w = sp.Weights.upload_u16(p, n, k_rows, 0) if enc == "u16" else sp.Weights.upload_delta(p, n, k_rows, 0, rows=m if m <= 8 else 0)
+            ncp = max(4, min(64, int(math.ceil(600e6 / w.nbytes))))
+            cps = [w] + [w.clone() for _ in range(ncp - 1)]
+            xh = sp.DeviceBuffer.from_numpy(sp.make_x_normal(0xC0FFEE ^ m, m, k_rows))
+            xq = sp.DeviceBuffer.from_numpy(sp.make_x_i8(0xC0FFEE ^ m, m, k_rows))
+            inv = sp.DeviceBuffer.from_numpy(np.full(m, 1.0 / 127.0, np.float32))
+            yb = sp.DeviceBuffer(4 * m * n_cols)
+            need = w.q8_workspace_bytes(m)
+            ws = sp.DeviceBuffer(need)
+            variants = (("int8_us", lambda c: c.gemv_i8(xq, m, yb, st)),
+                        ("int8_scaled_us", lambda c: c.gemv_i8_scaled(xq, inv, m, 1.0, yb, st)),
+                        ("quantising_fused_us", lambda c: c.gemv_q8(xh, 1, m, 1.0, yb, st)),
+                        ("quantising_workspace_us", lambda c: c.gemv_q8_ws(xh, 1, m, 1.0, yb, ws, need, st)))
+            r = {"K": k_rows, "N": n_cols, "S": s_nz, "enc": enc, "M": m}
+            for name, call in variants:
+                for c in cps:
+                    call(c)
+                st.sync()
+                best = None
+                for _ in range(3):
+                    t0 = time.perf_counter()
+                    done = 0
+                    while done < calls:
+                        for c in cps:
+                            call(c)
+                        done += ncp
+                    st.sync()
+                    us = (time.perf_counter() - t0) / done * 1e6
+                    best = us if best is None else min(best, us)
+                r[name] = round(best, 2)
+            rows.append(r)
+            for o in cps + [xh, xq, inv, yb, ws]:
+                o.free()
+    return {"rows": rows, "protocol": "host clock around %d calls + stream synchronise, best of three; one call = one or two launches on one stream, "
+                                      "rotating over device copies of the stream (HBM-cold)" % calls}
+
+
 def plans_leg(sp, n_shapes=12):
     """The launch-shape model against a bounded on-device search (sptmm_weights_tune), over seeded random shapes the model
     was never fitted on: K and N multiples of 256, 8-60 % nonzeros, both list encodings, a lone GEMV, a batched launch of 16
@@ -204,7 +253,7 @@ def plans_leg(sp, n_shapes=12):
         Wm, p, n = sp.generate_ternary(k_rows, n_cols, s_nz)
         for enc in ("u16", "delta"):
             for m, batch in ((1, 0), (1, 16), (4, 16)):
-                w = sp.Weights.upload_u16(p, n, k_rows, 0) if enc == "u16" else sp.Weights.upload_delta(p, n, k_rows, 0, rows=m)
+                w = sp.Weights.upload_u16(p, n, k_rows, 0) if enc == "u16" else sp.Weights.upload_delta(p, n, k_rows, 0, rows=m if m <= 8 else 0)
                 us_model, us_best, plan = w.tune(m, batch)
                 rows.append({"K": k_rows, "N": n_cols, "S": s_nz, "enc": enc, "M": m, "gemvs_per_launch": batch or 1, "split_k": w.info["split_k"],
                              "model_us": round(us_model, 3), "best_plan_us": round(us_best, 3), "model_over_best": round(us_model / us_best, 3),
@@ -228,7 +277,7 @@ def run(argv=None):
     ap.add_argument("--reps", type=int, default=0,
                     help="launches per timed loop of the legs (0: 1500, the headline shape's other encodings 4096); counter "
                          "runs under a profiler, where every launch is serialised, use a few dozen")
-    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,layer,cfg4,density,plans",
+    ap.add_argument("--legs", default="single,others,ceiling,cfg1,cfg2,cfg3,layer,cfg4,density,plans,q8",
                     help="extra legs besides the headline loop: single (one GEMV per launch: cold, warm, sync-each-call, four streams), "
                          "others (delta and i2s encodings at the headline shape), cfg1 (the same matrix at M=4), cfg2 (gap "
                          "stream with fp16 rows), cfg3 (decoder-layer shapes, M=1 and 4), cfg4 (K=13824 N=5120, M=1/8/16), "
@@ -236,6 +285,7 @@ def run(argv=None):
                          "issued in order / as a HIP graph, rotating over enough layers to stay HBM-cold), "
                          "density (the headline shape at 3.7-25 % nonzeros against i2s), "
                          "plans (the launch-shape model against sptmm_weights_tune over random shapes), "
+                         "q8 (the headline shape through the int8, scaled-int8 and quantising calls, one call at a time), "
                          "copy (4 launches of a 1 GiB copy kernel, for counter calibration), ceiling (a pure streaming "
                          "read of as many bytes as one step moves); profiling runs use --legs none or one leg")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
@@ -487,6 +537,7 @@ def run(argv=None):
         density = {"shapes": rows, "against_i2s": cross, "lists_beat_i2s_up_to_density_pct": max(wins) if wins else None}
 
     plans = plans_leg(sp) if "plans" in legs else None
+    quantising = quantising_leg(sp, st, K, N, S, calls=min(a.reps or 600, 600)) if "q8" in legs else None
 
     gbps = nbytes / us_gemv / 1e3
     traffic, traffic_src = None, None
@@ -522,6 +573,7 @@ def run(argv=None):
             "beats_i2s_batched_up_to_density_pct": density["lists_beat_i2s_up_to_density_pct"] if density else None,
         },
         "single_launch": single, "other_encodings": others, "configs": configs, "layer_sequence": layer_seq, "density_sweep": density, "launch_plans": plans,
+        "quantising_calls": quantising,
         "device": {"arch": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_src,
@@ -596,6 +648,10 @@ def final_line(full):
         summary["density_lists_over_i2s"] = {str(c["density_pct"]): c["lists_over_i2s"] for c in dn["against_i2s"]}
     if full.get("launch_plans"):
         summary["launch_plans_model_vs_tuned"] = full["launch_plans"]["summary"]
+    if full.get("quantising_calls"):
+        summary["quantising_calls_us"] = {"columns": ["int8", "int8_scaled", "quantising_fused", "quantising_workspace"]}
+        for r in full["quantising_calls"]["rows"]:
+            summary["quantising_calls_us"]["M%d_%s" % (r["M"], r["enc"])] = [r["int8_us"], r["int8_scaled_us"], r["quantising_fused_us"], r["quantising_workspace_us"]]
     out["summary"] = summary
     out["detail_file"] = full.get("detail_file")
     return json.dumps(out, ensure_ascii=False, separators=(",", ":"))
@@ -612,7 +668,7 @@ def main():
                 json.dump(full, f, ensure_ascii=False, indent=1)
         except OSError as e:  # a read-only tree: the tables still go to stderr
             print("bench.py: cannot write %s: %s" % (path, e), file=sys.stderr)
-    for leg in ("single_launch", "other_encodings", "configs", "layer_sequence", "density_sweep", "launch_plans"):
+    for leg in ("single_launch", "other_encodings", "configs", "layer_sequence", "density_sweep", "launch_plans", "quantising_calls"):
         if full.get(leg):
             print(json.dumps({leg: full[leg]}, ensure_ascii=False), file=sys.stderr)
     print(final_line(full), flush=True)

@@ -27,7 +27,7 @@ def test_final_line_of_a_full_run_is_short_and_keeps_the_contract():
     import bench
 
     full = json.load(open(os.path.join(ROOT, "tests", "golden", "bench_full_sample.json")))
-    for leg in ("single_launch", "other_encodings", "configs", "density_sweep", "cpu_baseline", "layer_sequence", "launch_plans"):
+    for leg in ("single_launch", "other_encodings", "configs", "density_sweep", "cpu_baseline", "layer_sequence", "launch_plans", "quantising_calls"):
         assert full.get(leg), leg
     assert len(json.dumps(full)) > 4 * LINE_LIMIT  # the sample really holds the tables
     line = bench.final_line(full)
