@@ -885,6 +885,9 @@ struct ListsBody {
         float back[MT];
 #pragma unroll
         for (int m = 0; m < MT; ++m) back[m] = QUANT == 1 ? qinv[m] : QUANT == 2 ? (m0 + m < p.M ? p.inv[m0 + m] : 0.f) : 0.f;
+        // rows quantised beforehand, matrix-unit epilogues: lane l writes row l & (MT - 1); its 1/s is fetched once, here
+        float inv_lane = 0.f;
+        if constexpr (QUANT == 2) inv_lane = m0 + (lane & (MT - 1)) < p.M ? p.inv[m0 + (lane & (MT - 1))] : 0.f;
         for (int it = 0; it < p.iters; ++it, task += task_step) {
             const bool active = task < p.tasks;
             const uint8_t *tb = tasks_base + (size_t)(active ? task : 0) * task_bytes;
@@ -1062,7 +1065,7 @@ struct ListsBody {
                             if (active && lane < (logL == 5 ? 16 : 8) && m0 + m < p.M) {
                                 const int col = (task << (6 - logL)) + (lane >> 3);
                                 if constexpr (QUANT != 0)
-                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)v * (QUANT == 1 ? qinv[m] : p.inv[m0 + m]) * p.w_scale;
+                                    Cf[(size_t)(m0 + m) * p.N + col] = (float)v * (QUANT == 1 ? qinv[m] : inv_lane) * p.w_scale;
                                 else
                                     C[(size_t)(m0 + m) * p.N + col] = v;
                             }
@@ -1100,7 +1103,7 @@ struct ListsBody {
                 if (p.W == 1) {
                     if (active && writer && m0 + m < p.M) {
                         const int cbase = task << (6 - logL);
-                        const float bk = QUANT == 1 ? qinv[m] : QUANT == 2 ? p.inv[m0 + m] : 0.f;
+                        const float bk = QUANT == 1 ? qinv[m] : QUANT == 2 ? inv_lane : 0.f;
 #pragma unroll
                         for (int x = 0; x < ND; ++x) {
                             if (x > 0 && logL >= 6) break;  // one column per task: tile 1 is already in t[0]
